@@ -1,0 +1,57 @@
+// Shared declarations of the host layer and the kernel launchers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <cstdio>
+
+// Error convention of the reference (QW/src/debug_utils.h:56-64): always on, stderr,
+// "ERROR: <message> (<file>:<line>)".
+#define MI_ERROR_FMT(fmt, ...) \
+    std::fprintf(stderr, "ERROR: " fmt " (%s:%d)\n", ##__VA_ARGS__, __FILE__, __LINE__)
+
+#define MI_HIP_OK(call)                                                          \
+    ([&]() -> bool {                                                             \
+        hipError_t e_ = (call);                                                  \
+        if (e_ != hipSuccess) {                                                  \
+            MI_ERROR_FMT("%s failed: %s", #call, hipGetErrorString(e_));         \
+            return false;                                                        \
+        }                                                                        \
+        return true;                                                             \
+    }())
+
+namespace mi {
+
+enum WeightKind : int { WK_F16 = 0, WK_Q4 = 4, WK_I8 = 8 };
+enum Epilogue : int { EPI_STORE = 0, EPI_ADD = 1 };
+
+struct DeviceInfo {
+    int  device = -1;
+    int  cus = 0;
+    char arch[64] = {0};
+};
+const DeviceInfo& device_info();
+
+// M rows of x (stride K) against one W; y rows have stride N.
+struct GemvCall {
+    const void* x = nullptr;      // fp16 [M,K]
+    const void* W = nullptr;      // fp16 [N,K] | int8 [N,K] | u8 [N,K/2]
+    const void* scale = nullptr;  // fp16 [N] (int8) | fp16 [N,K/32] (Q4) | null
+    void*       y = nullptr;      // fp16 [M,N]; read-modify-write for EPI_ADD
+    int M = 1, N = 0, K = 0;
+    WeightKind kind = WK_F16;
+    Epilogue   epi = EPI_STORE;
+};
+
+// gemv.hip
+bool launch_gemv(hipStream_t s, const GemvCall& c);
+bool launch_gate_up_silu(hipStream_t s, WeightKind kind, int N, int K, const void* x,
+                         const void* Wg, const void* sg, const void* Wu, const void* su, void* out);
+bool launch_dequant_int8(hipStream_t s, const void* q, const void* scale, int N, int K, void* w16);
+bool launch_unpack_q4(hipStream_t s, const void* p, int N, int K, void* w8);
+
+// gemm.hip: out[M,N] = x[M,K] W^T on MFMA with the dequant fused into the tile load.
+bool gemm_supported(WeightKind kind, int M, int N, int K);
+bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x,
+                 const void* W, const void* scale, void* out);
+
+}  // namespace mi

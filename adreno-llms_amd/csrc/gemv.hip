@@ -1,0 +1,496 @@
+// Batch-1 (and small-batch) GEMV kernels for gfx950: y[n] = sum_k x[k] * W[n,k] with fp16,
+// per-row int8 or block-32 Q4 weights, fp32 accumulation, fp16 output.
+//
+// Arithmetic contract.  The reference kernels (QW/kernels/gemv_m1.cl:366-462, 580-690,
+// LF/kernels/gemv_m1_int8.cl:32-79, LF/kernels/gemv_m1_q4.cl:45-123) give each of 64
+// work-items, in K-iteration j, one "pixel" of a row: 4 consecutive elements (fp16, int8)
+// or 8 (Q4); the item keeps one fp32 accumulator per row, and the 64 accumulators are
+// summed by a tree (t += t+s, s = 32..1).  These kernels evaluate exactly that sum, in that
+// order, so results are bit-identical to a literal evaluation of the reference kernels:
+// the 64 accumulators of a row are "virtual lanes", and one hardware lane owns VL
+// consecutive virtual lanes.  With VL = 4 a lane reads 16 bytes of int8/Q4 weights per
+// iteration (one global_load_dwordx4), 16 lanes cover a row-iteration and a 64-wide
+// wavefront works on 4 rows at once; VL = 2 and VL = 1 trade load width for more
+// wavefronts when N is small.  Tree steps with s >= VL are cross-lane adds inside the
+// 64/VL-lane group, steps with s < VL are adds between a lane's own accumulators.
+//
+// A lane's K positions do not depend on the row, so in the fixed-K kernels the lane loads
+// its slice of x once into registers and then streams rows: the inner loop issues only
+// weight loads (every byte of W is read exactly once, fully coalesced) and two VALU
+// operations per int8 weight (v_cvt_f32_i32 with a byte select, v_fma_mix_f32 taking x
+// straight from its fp16 register half).  No MFMA: at batch 1 the op is HBM-bound.
+#include "common.h"
+#include <hip/hip_fp16.h>
+
+namespace mi {
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = kWave * kWavesPerBlock;
+
+template <int KIND> struct WT;
+template <> struct WT<WK_F16> { static constexpr int EPV = 4, BPV = 8; };  // elements / bytes per virtual lane
+template <> struct WT<WK_I8>  { static constexpr int EPV = 4, BPV = 4; };
+template <> struct WT<WK_Q4>  { static constexpr int EPV = 8, BPV = 4; };
+
+__device__ __forceinline__ float lo_f(uint32_t p) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(p & 0xffffu)));
+}
+__device__ __forceinline__ float hi_f(uint32_t p) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(p >> 16)));
+}
+__device__ __forceinline__ float h_f(uint16_t h) { return __half2float(__ushort_as_half(h)); }
+__device__ __forceinline__ uint16_t f_h(float f) { return __half_as_ushort(__float2half_rn(f)); }
+
+// Two nibbles (bits 0-3 and 16-19 of v) -> two fp16 values (nibble - 8), exact:
+// 0x6400 | n is the half 1024 + n, and (1024 + n) - 1032 is exact.
+__device__ __forceinline__ uint32_t nib_pair(uint32_t v) {
+    uint32_t t = (v & 0x000F000Fu) | 0x64006400u;
+    __half2 h = __builtin_bit_cast(__half2, t);
+    h = __hsub2(h, __builtin_bit_cast(__half2, 0x64086408u));
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// One virtual lane, one K-iteration.  `scale` is used by Q4 only.
+template <int KIND>
+__device__ __forceinline__ float vlane_step(float acc, const uint32_t* w, const uint32_t* x, float scale) {
+    if constexpr (KIND == WK_F16) {
+        float d = lo_f(x[0]) * lo_f(w[0]);
+        d = fmaf(hi_f(x[0]), hi_f(w[0]), d);
+        d = fmaf(lo_f(x[1]), lo_f(w[1]), d);
+        d = fmaf(hi_f(x[1]), hi_f(w[1]), d);
+        return acc + d;
+    } else if constexpr (KIND == WK_I8) {
+        const uint32_t v = w[0];
+        const float w0 = static_cast<float>(static_cast<int8_t>(v & 0xffu));
+        const float w1 = static_cast<float>(static_cast<int8_t>((v >> 8) & 0xffu));
+        const float w2 = static_cast<float>(static_cast<int8_t>((v >> 16) & 0xffu));
+        const float w3 = static_cast<float>(static_cast<int8_t>(v >> 24));
+        float d = lo_f(x[0]) * w0;
+        d = fmaf(hi_f(x[0]), w1, d);
+        d = fmaf(lo_f(x[1]), w2, d);
+        d = fmaf(hi_f(x[1]), w3, d);
+        return acc + d;
+    } else {
+        const uint32_t v = w[0];
+        const uint32_t p04 = nib_pair(v), p15 = nib_pair(v >> 4);
+        const uint32_t p26 = nib_pair(v >> 8), p37 = nib_pair(v >> 12);
+        float d = lo_f(x[0]) * lo_f(p04);
+        d = fmaf(hi_f(x[0]), lo_f(p15), d);
+        d = fmaf(lo_f(x[1]), lo_f(p26), d);
+        d = fmaf(hi_f(x[1]), lo_f(p37), d);
+        d = fmaf(lo_f(x[2]), hi_f(p04), d);
+        d = fmaf(hi_f(x[2]), hi_f(p15), d);
+        d = fmaf(lo_f(x[3]), hi_f(p26), d);
+        d = fmaf(hi_f(x[3]), hi_f(p37), d);
+        return fmaf(d, scale, acc);
+    }
+}
+
+template <int ND> __device__ __forceinline__ void load_dwords(uint32_t* dst, const void* src) {
+    if constexpr (ND == 1) {
+        dst[0] = *static_cast<const uint32_t*>(src);
+    } else if constexpr (ND == 2) {
+        const uint2 v = *static_cast<const uint2*>(src);
+        dst[0] = v.x; dst[1] = v.y;
+    } else {
+        static_assert(ND % 4 == 0, "dword count");
+        #pragma unroll
+        for (int i = 0; i < ND / 4; ++i) {
+            const uint4 v = static_cast<const uint4*>(src)[i];
+            dst[4 * i] = v.x; dst[4 * i + 1] = v.y; dst[4 * i + 2] = v.z; dst[4 * i + 3] = v.w;
+        }
+    }
+}
+
+// The 64-virtual-lane tree of the reference, on VL accumulators per lane.
+template <int VL> __device__ __forceinline__ float reduce_row(float (&acc)[VL]) {
+    constexpr int LPR = kWave / VL;
+    #pragma unroll
+    for (int off = LPR / 2; off >= 1; off >>= 1) {
+        #pragma unroll
+        for (int v = 0; v < VL; ++v) acc[v] = acc[v] + __shfl_down(acc[v], off, LPR);
+    }
+    #pragma unroll
+    for (int s = VL / 2; s >= 1; s >>= 1) {
+        #pragma unroll
+        for (int v = 0; v < s; ++v) acc[v] = acc[v] + acc[v + s];
+    }
+    return acc[0];
+}
+
+template <int KIND, int EPI>
+__device__ __forceinline__ void epilogue(float sum, const uint16_t* sc, uint16_t* y, int row) {
+    if constexpr (KIND == WK_I8) {
+        const float s = h_f(sc[row]);
+        if constexpr (EPI == EPI_ADD) y[row] = f_h(fmaf(sum, s, h_f(y[row])));
+        else y[row] = f_h(sum * s);
+    } else {
+        if constexpr (EPI == EPI_ADD) y[row] = f_h(sum + h_f(y[row]));
+        else y[row] = f_h(sum);
+    }
+}
+
+// ---- K known at compile time: x lives in registers ---------------------------------
+template <int KIND, int KT, int VL, int EPI>
+__global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restrict__ x,
+                                                       const uint8_t* __restrict__ W,
+                                                       const uint16_t* __restrict__ sc,
+                                                       uint16_t* __restrict__ y, int N) {
+    using T = WT<KIND>;
+    constexpr int LPR = kWave / VL, RPW = VL;
+    constexpr int EIT = kWave * T::EPV;                 // elements per K-iteration
+    constexpr int NIT = (KT + EIT - 1) / EIT;
+    constexpr int XD = VL * T::EPV / 2;                 // x dwords per lane and iteration
+    constexpr int WD = VL * T::BPV / 4;                 // weight dwords per lane and iteration
+    constexpr int ROWB = KT / T::EPV * T::BPV;          // bytes per weight row
+    constexpr int ITB = kWave * T::BPV;                 // weight bytes per row and iteration
+
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int g = lane % LPR, r = lane / LPR;
+    const int koff = g * VL * T::EPV;
+    x += static_cast<size_t>(blockIdx.y) * KT;
+    y += static_cast<size_t>(blockIdx.y) * N;
+
+    uint32_t xr[NIT][XD];
+    #pragma unroll
+    for (int j = 0; j < NIT; ++j) {
+        if (j * EIT + koff < KT) load_dwords<XD>(xr[j], x + j * EIT + koff);
+        else {
+            #pragma unroll
+            for (int i = 0; i < XD; ++i) xr[j][i] = 0u;
+        }
+    }
+
+    const int nbatch = (N + RPW - 1) / RPW;
+    for (int rb = blockIdx.x * kWavesPerBlock + wave; rb < nbatch; rb += gridDim.x * kWavesPerBlock) {
+        const int row = rb * RPW + r;
+        const bool valid = row < N;
+        const int rowc = valid ? row : N - 1;
+        const uint8_t* wrow = W + static_cast<size_t>(rowc) * ROWB + koff / T::EPV * T::BPV;
+
+        uint32_t wr[NIT][WD];
+        float sf[NIT];
+        #pragma unroll
+        for (int j = 0; j < NIT; ++j) {
+            if (j * EIT + koff < KT) {
+                load_dwords<WD>(wr[j], wrow + j * ITB);
+                if constexpr (KIND == WK_Q4)
+                    sf[j] = h_f(sc[static_cast<size_t>(rowc) * (KT / 32) + j * 16 + (g * VL) / 4]);
+                else sf[j] = 0.0f;
+            }
+        }
+        float acc[VL];
+        #pragma unroll
+        for (int v = 0; v < VL; ++v) acc[v] = 0.0f;
+        #pragma unroll
+        for (int j = 0; j < NIT; ++j) {
+            if (j * EIT + koff < KT) {
+                #pragma unroll
+                for (int v = 0; v < VL; ++v)
+                    acc[v] = vlane_step<KIND>(acc[v], &wr[j][v * T::BPV / 4], &xr[j][v * T::EPV / 2], sf[j]);
+            }
+        }
+        const float sum = reduce_row<VL>(acc);
+        if (g == 0 && valid) epilogue<KIND, EPI>(sum, sc, y, row);
+    }
+}
+
+// ---- K known at run time: x is staged once per block in LDS ------------------------
+template <int KIND, int VL, int EPI>
+__global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict__ x,
+                                                     const uint8_t* __restrict__ W,
+                                                     const uint16_t* __restrict__ sc,
+                                                     uint16_t* __restrict__ y, int N, int K) {
+    using T = WT<KIND>;
+    constexpr int LPR = kWave / VL, RPW = VL;
+    constexpr int EIT = kWave * T::EPV;
+    constexpr int XD = VL * T::EPV / 2;
+    constexpr int WD = VL * T::BPV / 4;
+    constexpr int ITB = kWave * T::BPV;
+    extern __shared__ uint32_t xs[];                    // K/2 dwords of packed fp16
+
+    x += static_cast<size_t>(blockIdx.y) * K;
+    y += static_cast<size_t>(blockIdx.y) * N;
+    for (int i = threadIdx.x; i < K / 2; i += kBlock) xs[i] = reinterpret_cast<const uint32_t*>(x)[i];
+    __syncthreads();
+
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int g = lane % LPR, r = lane / LPR;
+    const int koff = g * VL * T::EPV;
+    const size_t rowb = static_cast<size_t>(K) / T::EPV * T::BPV;
+    const int nit = (K + EIT - 1) / EIT;
+    const int nbatch = (N + RPW - 1) / RPW;
+
+    for (int rb = blockIdx.x * kWavesPerBlock + wave; rb < nbatch; rb += gridDim.x * kWavesPerBlock) {
+        const int row = rb * RPW + r;
+        const bool valid = row < N;
+        const int rowc = valid ? row : N - 1;
+        const uint8_t* wrow = W + static_cast<size_t>(rowc) * rowb + koff / T::EPV * T::BPV;
+        const uint16_t* srow = sc + static_cast<size_t>(rowc) * (K / 32) + (g * VL) / 4;
+        float acc[VL];
+        #pragma unroll
+        for (int v = 0; v < VL; ++v) acc[v] = 0.0f;
+        #pragma unroll 4
+        for (int j = 0; j < nit; ++j) {
+            const int k = j * EIT + koff;
+            if (k < K) {
+                uint32_t wr[WD], xr[XD];
+                load_dwords<WD>(wr, wrow + static_cast<size_t>(j) * ITB);
+                #pragma unroll
+                for (int i = 0; i < XD; ++i) xr[i] = xs[k / 2 + i];
+                float sf = 0.0f;
+                if constexpr (KIND == WK_Q4) sf = h_f(srow[j * 16]);
+                #pragma unroll
+                for (int v = 0; v < VL; ++v)
+                    acc[v] = vlane_step<KIND>(acc[v], &wr[v * T::BPV / 4], &xr[v * T::EPV / 2], sf);
+            }
+        }
+        const float sum = reduce_row<VL>(acc);
+        if (g == 0 && valid) epilogue<KIND, EPI>(sum, sc, y, row);
+    }
+}
+
+// exp() of the SwiGLU epilogue: range reduction by ln2 in two parts and a degree-7 Horner
+// polynomial, built from fma/rint/ldexp only so that a host evaluation of the same
+// formula gives the same bits (the reference's native_exp has no defined precision,
+// SM/kernels/block_fused_int8.cl:229).
+__device__ __forceinline__ float exp_poly(float x) {
+    if (x > 88.0f) return __builtin_huge_valf();
+    if (x < -87.0f) return 0.0f;
+    const float n = rintf(x * 1.44269504088896341f);
+    float r = fmaf(n, -0.693145751953125f, x);
+    r = fmaf(n, -1.42860682030941723212e-6f, r);
+    float p = 1.0f / 5040.0f;
+    p = fmaf(p, r, 1.0f / 720.0f);
+    p = fmaf(p, r, 1.0f / 120.0f);
+    p = fmaf(p, r, 1.0f / 24.0f);
+    p = fmaf(p, r, 1.0f / 6.0f);
+    p = fmaf(p, r, 0.5f);
+    p = fmaf(p, r, 1.0f);
+    p = fmaf(p, r, 1.0f);
+    return ldexpf(p, static_cast<int>(n));
+}
+
+// out[c] = fp16( silu(g) * u ), g and u the two row sums (scaled for int8).
+// SM/kernels/block_fused_int8.cl:176-236, SM/kernels/block_fused.cl:473-526.
+template <int KIND, int VL>
+__global__ __launch_bounds__(kBlock) void gate_up_silu_any_k(const uint16_t* __restrict__ x,
+                                                             const uint8_t* __restrict__ Wg,
+                                                             const uint16_t* __restrict__ sg,
+                                                             const uint8_t* __restrict__ Wu,
+                                                             const uint16_t* __restrict__ su,
+                                                             uint16_t* __restrict__ out, int N, int K) {
+    using T = WT<KIND>;
+    constexpr int LPR = kWave / VL, RPW = VL;
+    constexpr int EIT = kWave * T::EPV;
+    constexpr int XD = VL * T::EPV / 2;
+    constexpr int WD = VL * T::BPV / 4;
+    constexpr int ITB = kWave * T::BPV;
+    extern __shared__ uint32_t xs[];
+    for (int i = threadIdx.x; i < K / 2; i += kBlock) xs[i] = reinterpret_cast<const uint32_t*>(x)[i];
+    __syncthreads();
+
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int g = lane % LPR, r = lane / LPR;
+    const int koff = g * VL * T::EPV;
+    const size_t rowb = static_cast<size_t>(K) / T::EPV * T::BPV;
+    const int nit = (K + EIT - 1) / EIT;
+    const int nbatch = (N + RPW - 1) / RPW;
+
+    for (int rb = blockIdx.x * kWavesPerBlock + wave; rb < nbatch; rb += gridDim.x * kWavesPerBlock) {
+        const int row = rb * RPW + r;
+        const bool valid = row < N;
+        const int rowc = valid ? row : N - 1;
+        const size_t off = static_cast<size_t>(rowc) * rowb + koff / T::EPV * T::BPV;
+        float ag[VL], au[VL];
+        #pragma unroll
+        for (int v = 0; v < VL; ++v) { ag[v] = 0.0f; au[v] = 0.0f; }
+        #pragma unroll 2
+        for (int j = 0; j < nit; ++j) {
+            const int k = j * EIT + koff;
+            if (k < K) {
+                uint32_t wg[WD], wu[WD], xr[XD];
+                load_dwords<WD>(wg, Wg + off + static_cast<size_t>(j) * ITB);
+                load_dwords<WD>(wu, Wu + off + static_cast<size_t>(j) * ITB);
+                #pragma unroll
+                for (int i = 0; i < XD; ++i) xr[i] = xs[k / 2 + i];
+                #pragma unroll
+                for (int v = 0; v < VL; ++v) {
+                    ag[v] = vlane_step<KIND>(ag[v], &wg[v * T::BPV / 4], &xr[v * T::EPV / 2], 0.0f);
+                    au[v] = vlane_step<KIND>(au[v], &wu[v * T::BPV / 4], &xr[v * T::EPV / 2], 0.0f);
+                }
+            }
+        }
+        float gs = reduce_row<VL>(ag);
+        float us = reduce_row<VL>(au);
+        if (g == 0 && valid) {
+            if constexpr (KIND == WK_I8) { gs = gs * h_f(sg[row]); us = us * h_f(su[row]); }
+            out[row] = f_h((gs / (1.0f + exp_poly(-gs))) * us);
+        }
+    }
+}
+
+// w16[n,k] = fp16(f32(q[n,k]) * f32(scale[n]))   (LV/kernels/lfm2_ops.cl:731-743)
+__global__ __launch_bounds__(256) void dequant_int8_kernel(const int8_t* __restrict__ q,
+                                                           const uint16_t* __restrict__ sc,
+                                                           uint16_t* __restrict__ w16, size_t total, int K) {
+    for (size_t i = blockIdx.x * 256ull + threadIdx.x; i < total; i += gridDim.x * 256ull)
+        w16[i] = f_h(static_cast<float>(q[i]) * h_f(sc[i / K]));
+}
+
+// w8[n,k] = nibble(n,k) - 8   (LF/kernels/gemv_m1_q4.cl:31-40)
+__global__ __launch_bounds__(256) void unpack_q4_kernel(const uint8_t* __restrict__ p,
+                                                        int8_t* __restrict__ w8, size_t nbytes) {
+    for (size_t i = blockIdx.x * 256ull + threadIdx.x; i < nbytes; i += gridDim.x * 256ull) {
+        const uint8_t b = p[i];
+        w8[2 * i] = static_cast<int8_t>(static_cast<int>(b & 0xF) - 8);
+        w8[2 * i + 1] = static_cast<int8_t>(static_cast<int>(b >> 4) - 8);
+    }
+}
+
+// ---- launch side -------------------------------------------------------------------
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// Widest lane tile that still gives every SIMD of the chip a wavefront; when no tile
+// reaches that, the narrowest one (most wavefronts).  A tile of VL fits when a lane's
+// VL virtual lanes are whole in the K tail.
+int pick_vl(WeightKind kind, int M, int N, int K) {
+    const int epv = kind == WK_Q4 ? 8 : 4;
+    const int max_vl = kind == WK_F16 ? 2 : 4;
+    const long waves_wanted = 4L * device_info().cus;
+    int narrowest = 1;
+    for (int vl = max_vl; vl >= 1; vl >>= 1) {
+        if (K % (vl * epv) != 0) continue;
+        narrowest = vl;
+        if (static_cast<long>(M) * ((N + vl - 1) / vl) >= waves_wanted) return vl;
+    }
+    return narrowest;
+}
+
+dim3 grid_for(int M, int N, int vl) {
+    const int nbatch = (N + vl - 1) / vl;
+    const int blocks = (nbatch + kWavesPerBlock - 1) / kWavesPerBlock;
+    const int cap = device_info().cus * 8;                  // 32 wavefronts per CU
+    return dim3(blocks < cap ? blocks : cap, M, 1);
+}
+
+template <int KIND, int VL, int EPI>
+bool launch_kind_vl(hipStream_t s, const GemvCall& c) {
+    const auto* x = static_cast<const uint16_t*>(c.x);
+    const auto* W = static_cast<const uint8_t*>(c.W);
+    const auto* sc = static_cast<const uint16_t*>(c.scale);
+    auto* y = static_cast<uint16_t*>(c.y);
+    const dim3 grid = grid_for(c.M, c.N, VL);
+#define MI_FIXED(KT)                                                                          \
+    case KT:                                                                                  \
+        hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI>), grid, dim3(kBlock), 0, s, x, W, \
+                           sc, y, c.N);                                                       \
+        break;
+    switch (c.K) {
+        MI_FIXED(576)
+        MI_FIXED(896)
+        MI_FIXED(1024)
+        MI_FIXED(1536)
+        MI_FIXED(4864)
+        default: {
+            const size_t lds = static_cast<size_t>(c.K) * 2;
+            hipLaunchKernelGGL((gemv_any_k<KIND, VL, EPI>), grid, dim3(kBlock), lds, s, x, W, sc, y,
+                               c.N, c.K);
+        }
+    }
+#undef MI_FIXED
+    return MI_HIP_OK(hipGetLastError());
+}
+
+template <int KIND, int EPI>
+bool launch_kind(hipStream_t s, const GemvCall& c, int vl) {
+    if constexpr (KIND != WK_F16) {
+        if (vl == 4) return launch_kind_vl<KIND, 4, EPI>(s, c);
+    }
+    if (vl == 2) return launch_kind_vl<KIND, 2, EPI>(s, c);
+    return launch_kind_vl<KIND, 1, EPI>(s, c);
+}
+
+}  // namespace
+
+bool launch_gemv(hipStream_t s, const GemvCall& c) {
+    const int epv = c.kind == WK_Q4 ? 32 : 4;               // Q4 needs whole scale blocks
+    if (c.M < 1 || c.N < 1 || c.K < 1 || c.K % epv != 0) {
+        MI_ERROR_FMT("gemv: unsupported shape M=%d N=%d K=%d (K must be a multiple of %d)", c.M, c.N,
+                     c.K, epv);
+        return false;
+    }
+    if (c.K > 32768 || c.M > 65535) {
+        MI_ERROR_FMT("gemv: K=%d or M=%d beyond the supported range", c.K, c.M);
+        return false;
+    }
+    if (!c.x || !c.W || !c.y || !aligned(c.x, 16) || !aligned(c.W, 16) || !aligned(c.y, 2) ||
+        (c.M > 1 && (static_cast<size_t>(c.K) * 2) % 16 != 0) ||
+        (c.kind != WK_F16 && (!c.scale || !aligned(c.scale, 2)))) {
+        MI_ERROR_FMT("gemv: null or misaligned operand (x and W need 16-byte alignment)");
+        return false;
+    }
+    const int vl = pick_vl(c.kind, c.M, c.N, c.K);
+    const bool add = c.epi == EPI_ADD;
+    switch (c.kind) {
+        case WK_F16: return add ? launch_kind<WK_F16, EPI_ADD>(s, c, vl) : launch_kind<WK_F16, EPI_STORE>(s, c, vl);
+        case WK_I8:  return add ? launch_kind<WK_I8, EPI_ADD>(s, c, vl) : launch_kind<WK_I8, EPI_STORE>(s, c, vl);
+        case WK_Q4:  return add ? launch_kind<WK_Q4, EPI_ADD>(s, c, vl) : launch_kind<WK_Q4, EPI_STORE>(s, c, vl);
+    }
+    return false;
+}
+
+bool launch_gate_up_silu(hipStream_t s, WeightKind kind, int N, int K, const void* x, const void* Wg,
+                         const void* sg, const void* Wu, const void* su, void* out) {
+    if (kind == WK_Q4 || N < 1 || K < 4 || K % 4 != 0 || K > 32768) {
+        MI_ERROR_FMT("gate_up_silu: unsupported kind=%d N=%d K=%d", static_cast<int>(kind), N, K);
+        return false;
+    }
+    if (!aligned(x, 16) || !aligned(Wg, 16) || !aligned(Wu, 16)) {
+        MI_ERROR_FMT("gate_up_silu: x and W must be 16-byte aligned");
+        return false;
+    }
+    const int vl = pick_vl(kind, 1, N, K);
+    const dim3 grid = grid_for(1, N, vl);
+    const size_t lds = static_cast<size_t>(K) * 2;
+    const auto* xp = static_cast<const uint16_t*>(x);
+    const auto* g8 = static_cast<const uint8_t*>(Wg);
+    const auto* u8 = static_cast<const uint8_t*>(Wu);
+    const auto* sgp = static_cast<const uint16_t*>(sg);
+    const auto* sup = static_cast<const uint16_t*>(su);
+    auto* o = static_cast<uint16_t*>(out);
+#define MI_GUS(KIND, VL) \
+    hipLaunchKernelGGL((gate_up_silu_any_k<KIND, VL>), grid, dim3(kBlock), lds, s, xp, g8, sgp, u8, sup, o, N, K)
+    if (kind == WK_I8) {
+        if (vl == 4) MI_GUS(WK_I8, 4); else if (vl == 2) MI_GUS(WK_I8, 2); else MI_GUS(WK_I8, 1);
+    } else {
+        if (vl >= 2) MI_GUS(WK_F16, 2); else MI_GUS(WK_F16, 1);
+    }
+#undef MI_GUS
+    return MI_HIP_OK(hipGetLastError());
+}
+
+bool launch_dequant_int8(hipStream_t s, const void* q, const void* scale, int N, int K, void* w16) {
+    if (N < 1 || K < 1) { MI_ERROR_FMT("dequant_int8: bad shape N=%d K=%d", N, K); return false; }
+    const size_t total = static_cast<size_t>(N) * K;
+    const size_t blocks = (total + 255) / 256;
+    const unsigned grid = static_cast<unsigned>(blocks < 65536 ? blocks : 65536);
+    hipLaunchKernelGGL(dequant_int8_kernel, dim3(grid), dim3(256), 0, s, static_cast<const int8_t*>(q),
+                       static_cast<const uint16_t*>(scale), static_cast<uint16_t*>(w16), total, K);
+    return MI_HIP_OK(hipGetLastError());
+}
+
+bool launch_unpack_q4(hipStream_t s, const void* p, int N, int K, void* w8) {
+    if (N < 1 || K < 2 || K % 2) { MI_ERROR_FMT("unpack_q4: bad shape N=%d K=%d", N, K); return false; }
+    const size_t nbytes = static_cast<size_t>(N) * (K / 2);
+    const size_t blocks = (nbytes + 255) / 256;
+    const unsigned grid = static_cast<unsigned>(blocks < 65536 ? blocks : 65536);
+    hipLaunchKernelGGL(unpack_q4_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint8_t*>(p),
+                       static_cast<int8_t*>(w8), nbytes);
+    return MI_HIP_OK(hipGetLastError());
+}
+
+}  // namespace mi

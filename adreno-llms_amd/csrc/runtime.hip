@@ -1,0 +1,277 @@
+// Host layer behind the C ABI: device plumbing, the weight registry and the
+// `pytorch_linear` dispatcher (QW/src/utils.cpp:758-823, LF/src/utils.cpp:1263-1374).
+#include "../../include/mi_linear.h"
+#include "common.h"
+
+#include <cstring>
+#include <mutex>
+#include <unordered_map>
+
+namespace mi {
+namespace {
+
+DeviceInfo g_dev;
+bool g_inited = false;
+int g_gemm_mode = 0;
+
+// Side table W pointer -> {kind, scale, N, K}; the counterpart of s_int8_aux / s_q4_aux
+// (LF/src/utils.cpp:194-231).  The reference is single threaded and takes no lock; a
+// mutex costs nothing here and lets several host threads drive different streams.
+struct Entry {
+    WeightKind kind;
+    const void* scale;
+    int N, K;
+};
+std::unordered_map<const void*, Entry> g_registry;
+std::mutex g_registry_mu;
+
+bool ensure_init() {
+    if (g_inited) return true;
+    return mi_init(0) == 1;
+}
+
+bool lookup(const void* W, Entry* out) {
+    std::lock_guard<std::mutex> lk(g_registry_mu);
+    auto it = g_registry.find(W);
+    if (it == g_registry.end()) return false;
+    *out = it->second;
+    return true;
+}
+
+bool resolve(const char* who, const void* W, int N, int K, Entry* e) {
+    if (!lookup(W, e)) {
+        *e = Entry{WK_F16, nullptr, N, K};
+        return true;
+    }
+    if (e->N != N || e->K != K) {
+        // The reference's registration comment: "N, K ... must match the GEMV call site
+        // exactly" (LF/src/utils.h:126-128).
+        MI_ERROR_FMT("%s: W registered as [%d,%d] but called with N=%d K=%d", who, e->N, e->K, N, K);
+        return false;
+    }
+    return true;
+}
+
+inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
+
+}  // namespace
+
+const DeviceInfo& device_info() { return g_dev; }
+
+}  // namespace mi
+
+using namespace mi;
+
+extern "C" {
+
+int mi_init(int device) {
+    int count = 0;
+    if (!MI_HIP_OK(hipGetDeviceCount(&count))) return 0;
+    if (device < 0 || device >= count) {
+        MI_ERROR_FMT("mi_init: device %d not present (%d devices)", device, count);
+        return 0;
+    }
+    if (!MI_HIP_OK(hipSetDevice(device))) return 0;
+    hipDeviceProp_t prop;
+    if (!MI_HIP_OK(hipGetDeviceProperties(&prop, device))) return 0;
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        MI_ERROR_FMT("mi_init: device %d is %s; this library holds gfx950 code only", device,
+                     prop.gcnArchName);
+        return 0;
+    }
+    g_dev.device = device;
+    g_dev.cus = prop.multiProcessorCount;
+    std::snprintf(g_dev.arch, sizeof(g_dev.arch), "%s", prop.gcnArchName);
+    g_inited = true;
+    return 1;
+}
+
+const char* mi_device_arch(void) { return g_dev.arch; }
+int mi_device_cus(void) { return g_dev.cus; }
+
+void* mi_malloc(size_t bytes) {
+    if (!ensure_init()) return nullptr;
+    void* p = nullptr;
+    if (!MI_HIP_OK(hipMalloc(&p, bytes ? bytes : 1))) return nullptr;
+    return p;
+}
+
+int mi_free(void* p) {
+    if (!p) return 1;
+    mi_unregister_weight(p);
+    return MI_HIP_OK(hipFree(p)) ? 1 : 0;
+}
+
+int mi_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
+    if (!MI_HIP_OK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)))) return 0;
+    return MI_HIP_OK(hipStreamSynchronize(as_stream(stream))) ? 1 : 0;
+}
+
+int mi_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream) {
+    if (!MI_HIP_OK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(stream)))) return 0;
+    return MI_HIP_OK(hipStreamSynchronize(as_stream(stream))) ? 1 : 0;
+}
+
+int mi_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream) {
+    return MI_HIP_OK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream))) ? 1 : 0;
+}
+
+int mi_memset(void* dst, int byte, size_t bytes, void* stream) {
+    return MI_HIP_OK(hipMemsetAsync(dst, byte, bytes, as_stream(stream))) ? 1 : 0;
+}
+
+void* mi_stream_create(void) {
+    if (!ensure_init()) return nullptr;
+    hipStream_t s = nullptr;
+    if (!MI_HIP_OK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking))) return nullptr;
+    return s;
+}
+
+int mi_stream_destroy(void* s) { return s ? (MI_HIP_OK(hipStreamDestroy(as_stream(s))) ? 1 : 0) : 1; }
+int mi_stream_sync(void* s) { return MI_HIP_OK(hipStreamSynchronize(as_stream(s))) ? 1 : 0; }
+
+void* mi_event_create(void) {
+    if (!ensure_init()) return nullptr;
+    hipEvent_t e = nullptr;
+    if (!MI_HIP_OK(hipEventCreate(&e))) return nullptr;
+    return e;
+}
+int mi_event_destroy(void* e) { return e ? (MI_HIP_OK(hipEventDestroy(static_cast<hipEvent_t>(e))) ? 1 : 0) : 1; }
+int mi_event_record(void* e, void* s) {
+    return MI_HIP_OK(hipEventRecord(static_cast<hipEvent_t>(e), as_stream(s))) ? 1 : 0;
+}
+int mi_event_sync(void* e) { return MI_HIP_OK(hipEventSynchronize(static_cast<hipEvent_t>(e))) ? 1 : 0; }
+float mi_event_elapsed_ms(void* a, void* b) {
+    float ms = -1.0f;
+    if (!MI_HIP_OK(hipEventElapsedTime(&ms, static_cast<hipEvent_t>(a), static_cast<hipEvent_t>(b)))) return -1.0f;
+    return ms;
+}
+
+// ---- registry --------------------------------------------------------------------
+
+int mi_register_int8_weight(const void* W, const void* scale, int N, int K) {
+    if (!W || !scale || N <= 0 || K <= 0) return 0;          // LF/src/utils.cpp:358
+    std::lock_guard<std::mutex> lk(g_registry_mu);
+    g_registry[W] = Entry{WK_I8, scale, N, K};
+    return 1;
+}
+
+int mi_register_q4_weight(const void* W, const void* scale, int N, int K) {
+    if (!W || !scale || N <= 0 || K <= 0) return 0;          // LF/src/utils.cpp:585
+    if (K % 32 != 0) {
+        // the quantizer refuses such a K (LF/scripts/quantize_q4.py:68-69)
+        MI_ERROR_FMT("mi_register_q4_weight: K=%d is not a multiple of the block size 32", K);
+        return 0;
+    }
+    std::lock_guard<std::mutex> lk(g_registry_mu);
+    g_registry[W] = Entry{WK_Q4, scale, N, K};
+    return 1;
+}
+
+int mi_unregister_weight(const void* W) {
+    std::lock_guard<std::mutex> lk(g_registry_mu);
+    return g_registry.erase(W) ? 1 : 0;
+}
+
+int mi_weight_kind(const void* W) {
+    Entry e;
+    return lookup(W, &e) ? static_cast<int>(e.kind) : 0;
+}
+
+void mi_set_gemm_mode(int mode) { g_gemm_mode = mode; }
+
+// ---- hot path --------------------------------------------------------------------
+
+int mi_linear(void* stream, int M, int N, int K, const void* x, const void* W, void* out) {
+    if (!ensure_init()) return 0;
+    if (M <= 0 || N <= 0 || K <= 0 || !x || !W || !out) {
+        MI_ERROR_FMT("mi_linear: bad argument (M=%d N=%d K=%d x=%p W=%p out=%p)", M, N, K, x, W, out);
+        return 0;
+    }
+    Entry e;
+    if (!resolve("mi_linear", W, N, K, &e)) return 0;
+    // M > 1: a real contraction goes to the MFMA GEMM; small batches, and every batch in
+    // mode 1, run the GEMV once per row of x, as the reference's quantised prefill does.
+    if (M >= 16 && g_gemm_mode == 0 && gemm_supported(e.kind, M, N, K))
+        return launch_gemm(as_stream(stream), e.kind, M, N, K, x, W, e.scale, out) ? 1 : 0;
+    GemvCall c;
+    c.x = x; c.W = W; c.scale = e.scale; c.y = out;
+    c.M = M; c.N = N; c.K = K; c.kind = e.kind; c.epi = EPI_STORE;
+    return launch_gemv(as_stream(stream), c) ? 1 : 0;
+}
+
+int mi_linear_batch(void* stream, const mi_linear_call* calls, int n) {
+    if (!calls || n < 0) { MI_ERROR_FMT("mi_linear_batch: bad argument"); return 0; }
+    for (int i = 0; i < n; ++i) {
+        const mi_linear_call& c = calls[i];
+        if (!mi_linear(stream, c.M, c.N, c.K, c.x, c.W, c.out)) return i;
+    }
+    return n;
+}
+
+int mi_graph_begin(void* stream) {
+    if (!ensure_init()) return 0;
+    if (!stream) { MI_ERROR_FMT("mi_graph_begin: needs a stream made by mi_stream_create"); return 0; }
+    return MI_HIP_OK(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal)) ? 1 : 0;
+}
+
+void* mi_graph_end(void* stream) {
+    hipGraph_t g = nullptr;
+    if (!MI_HIP_OK(hipStreamEndCapture(as_stream(stream), &g)) || !g) return nullptr;
+    hipGraphExec_t exec = nullptr;
+    const bool ok = MI_HIP_OK(hipGraphInstantiate(&exec, g, nullptr, nullptr, 0));
+    hipGraphDestroy(g);
+    return ok ? exec : nullptr;
+}
+
+int mi_graph_launch(void* graph, void* stream) {
+    if (!graph) { MI_ERROR_FMT("mi_graph_launch: null graph"); return 0; }
+    return MI_HIP_OK(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), as_stream(stream))) ? 1 : 0;
+}
+
+int mi_graph_destroy(void* graph) {
+    return graph ? (MI_HIP_OK(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph))) ? 1 : 0) : 1;
+}
+
+int mi_linear_add(void* stream, int M, int N, int K, const void* x, const void* W, void* residual) {
+    if (!ensure_init()) return 0;
+    if (M != 1) return 0;                                     // predicate miss, not an error
+    if (N <= 0 || K <= 0 || !x || !W || !residual) {
+        MI_ERROR_FMT("mi_linear_add: bad argument (N=%d K=%d)", N, K);
+        return 0;
+    }
+    Entry e;
+    if (!resolve("mi_linear_add", W, N, K, &e)) return 0;
+    GemvCall c;
+    c.x = x; c.W = W; c.scale = e.scale; c.y = residual;
+    c.M = 1; c.N = N; c.K = K; c.kind = e.kind; c.epi = EPI_ADD;
+    return launch_gemv(as_stream(stream), c) ? 1 : 0;
+}
+
+int mi_linear_gate_up_silu(void* stream, int N, int K, const void* x, const void* Wg, const void* Wu,
+                           void* out) {
+    if (!ensure_init()) return 0;
+    if (N <= 0 || K <= 0 || !x || !Wg || !Wu || !out) {
+        MI_ERROR_FMT("mi_linear_gate_up_silu: bad argument (N=%d K=%d)", N, K);
+        return 0;
+    }
+    Entry eg, eu;
+    if (!resolve("mi_linear_gate_up_silu", Wg, N, K, &eg)) return 0;
+    if (!resolve("mi_linear_gate_up_silu", Wu, N, K, &eu)) return 0;
+    if (eg.kind != eu.kind || eg.kind == WK_Q4) return 0;     // predicate miss
+    return launch_gate_up_silu(as_stream(stream), eg.kind, N, K, x, Wg, eg.scale, Wu, eu.scale, out) ? 1 : 0;
+}
+
+int mi_dequant_int8_to_fp16(void* stream, const void* W, const void* scale, int N, int K, void* w16) {
+    if (!ensure_init()) return 0;
+    if (!W || !scale || !w16) { MI_ERROR_FMT("mi_dequant_int8_to_fp16: null argument"); return 0; }
+    return launch_dequant_int8(as_stream(stream), W, scale, N, K, w16) ? 1 : 0;
+}
+
+int mi_unpack_q4_to_int8(void* stream, const void* W, int N, int K, void* w8) {
+    if (!ensure_init()) return 0;
+    if (!W || !w8) { MI_ERROR_FMT("mi_unpack_q4_to_int8: null argument"); return 0; }
+    return launch_unpack_q4(as_stream(stream), W, N, K, w8) ? 1 : 0;
+}
+
+}  // extern "C"

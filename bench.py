@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul path on one MI355X.
+
+A step is one decode-step matmul sweep of a Qwen2.5-0.5B-shaped model at batch 1 with
+per-row int8 weights: 24 layers x {q, k, v, o, gate, up, down} + lm_head = 169 calls of
+pytorch_linear, enqueued in order on one stream (weights, activations and outputs are
+resident in HBM before the timed region starts).  `value` is the algorithmic bytes of
+the sweep (weights + scales, 494 873 344 B) divided by the time per step.
+
+Also reported on the same JSON line:
+  roofline     - the lm_head int8 GEMV kernel alone (W[151936x896], 136 744 192 algorithmic
+                 bytes per launch), timed with HIP events on the launch stream over a run of
+                 launches that rotates through enough weight copies to exceed the 256 MB
+                 last-level cache, so every launch streams from HBM;
+  cpu_baseline - the CPU oracle (a C restatement of the reference kernels, OpenMP over rows)
+                 on a bounded sample of the same sweep, on the host cores of this box;
+  detail       - per-config figures (int8 / Q4 / fp16 GEMV shapes).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+H, INTER, KV, VOCAB, LAYERS = 896, 4864, 128, 151936, 24
+LAYER_SHAPES = [("q", H, H), ("k", KV, H), ("v", KV, H), ("o", H, H),
+                ("gate", INTER, H), ("up", INTER, H), ("down", H, INTER)]
+HBM_PEAK_GBS = 8000.0
+
+
+def algo_bytes_i8(N, K):
+    return N * K + 2 * N + 2 * K + 2 * N          # weights + scales + x + y
+
+
+def algo_bytes_q4(N, K):
+    return N * K // 2 + 2 * N * (K // 32) + 2 * K + 2 * N
+
+
+def algo_bytes_f16(N, K):
+    return 2 * N * K + 2 * K + 2 * N
+
+
+def time_region(mil, queue, fn, reps):
+    e0, e1 = mil.Event(), mil.Event()
+    queue.finish()
+    e0.record(queue)
+    for _ in range(reps):
+        fn()
+    e1.record(queue)
+    e1.synchronize()
+    queue.finish()
+    return e0.elapsed_ms(e1) / reps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-detail", action="store_true", help="skip the per-config detail runs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    mil = importlib.import_module("adreno-llms_amd")
+    assert mil.lib().mi_init(0) == 1, "bench: no gfx950 device"
+    queue = mil.Queue()
+    t_setup = time.time()
+
+    # ---- synthetic model: W ~ N(0, 0.02) fp16, quantised per row to int8 ------------------
+    def make_i8(seed, N, K):
+        w = mil.synth_normal_f16(seed, 0.02, (N, K))
+        q, s = mil.quantize_int8(w)
+        qb, sb = mil.Buffer.from_host(q), mil.Buffer.from_host(s)
+        assert mil.nnopt_register_int8_weight(qb, sb, N, K)
+        return qb, sb, (q, s)
+
+    keep, calls = [], []
+    x_h = mil.Buffer.from_host(mil.synth_normal_f16(1, 1.0, (H,)))
+    x_i = mil.Buffer.from_host(mil.synth_normal_f16(2, 1.0, (INTER,)))
+    outs = {n: mil.Buffer(N * 2) for n, N, _ in LAYER_SHAPES}
+    logits = mil.Buffer(VOCAB * 2)
+    sweep_bytes = 0
+    host_layer0 = {}
+    for layer in range(LAYERS):
+        for j, (name, N, K) in enumerate(LAYER_SHAPES):
+            qb, sb, host = make_i8(1000 + layer * 16 + j, N, K)
+            keep += [qb, sb]
+            if layer == 0:
+                host_layer0[name] = host
+            calls.append((1, N, K, x_i if K == INTER else x_h, qb, outs[name]))
+            sweep_bytes += N * K + 2 * N
+    lm_q, lm_s, lm_host = make_i8(7, VOCAB, H)
+    calls.append((1, VOCAB, H, x_h, lm_q, logits))
+    sweep_bytes += VOCAB * H + 2 * VOCAB
+    assert sweep_bytes == 494873344, sweep_bytes
+    call_arr = mil.make_calls(calls)
+    setup_s = time.time() - t_setup
+
+    # ---- the sweep: stream launches and graph replay --------------------------------------
+    def sweep_stream():
+        n = mil.linear_batch(queue, call_arr)
+        assert n == len(call_arr)
+
+    for _ in range(args.warmup):
+        sweep_stream()
+    ms_stream = time_region(mil, queue, sweep_stream, args.steps)
+
+    with mil.Graph(queue) as graph:
+        sweep_stream()
+    for _ in range(args.warmup):
+        graph.launch()
+    ms_graph = time_region(mil, queue, graph.launch, args.steps)
+
+    launch_mode = "hip_graph" if ms_graph < ms_stream else "stream"
+    ms_step = min(ms_graph, ms_stream)
+    value = sweep_bytes / (ms_step * 1e-3) / 1e9
+
+    # ---- roofline of the dominant kernel: lm_head int8 GEMV, cold ---------------------------
+    copies = [(lm_q, lm_s)]
+    for c in range(2):                       # 3 x 136 MB > 256 MB of last-level cache
+        qb, sb = mil.Buffer(VOCAB * H), mil.Buffer(VOCAB * 2)
+        mil.lib().mi_memcpy_d2d(qb.ptr, lm_q.ptr, VOCAB * H, queue.handle)
+        mil.lib().mi_memcpy_d2d(sb.ptr, lm_s.ptr, VOCAB * 2, queue.handle)
+        assert mil.nnopt_register_int8_weight(qb, sb, VOCAB, H)
+        copies.append((qb, sb))
+    queue.finish()
+    lm_calls = mil.make_calls([(1, VOCAB, H, x_h, copies[i % 3][0], logits) for i in range(30)])
+    for _ in range(2):
+        mil.linear_batch(queue, lm_calls)
+    ms_lm = time_region(mil, queue, lambda: mil.linear_batch(queue, lm_calls), 10) / 30
+    lm_bytes = algo_bytes_i8(VOCAB, H)
+    achieved = lm_bytes / (ms_lm * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": "gemv int8 K=896 (lm_head, N=151936)", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": None, "us_per_launch": round(ms_lm * 1e3, 2), "bytes_per_launch": lm_bytes}
+
+    # ---- per-config detail -------------------------------------------------------------------
+    detail = {"decode_step_us_stream": round(ms_stream * 1e3, 1), "decode_step_us_graph": round(ms_graph * 1e3, 1),
+              "setup_s": round(setup_s, 1)}
+    if not args.no_detail:
+        def cold_gemv(kind, N, K, reps_pool):
+            """us per launch over a pool of distinct weights larger than the last-level cache."""
+            w = mil.synth_normal_f16(99, 0.02, (N, K))
+            if kind == "i8":
+                a, b = mil.quantize_int8(w)
+                nbytes = algo_bytes_i8(N, K)
+            elif kind == "q4":
+                a, b = mil.quantize_q4(w)
+                nbytes = algo_bytes_q4(N, K)
+            else:
+                a, b = w, None
+                nbytes = algo_bytes_f16(N, K)
+            pool = []
+            npool = max(3, min(reps_pool, int(600e6 // a.nbytes) + 1))
+            for _ in range(npool):
+                wb = mil.Buffer.from_host(a)
+                sb = mil.Buffer.from_host(b) if b is not None else None
+                if kind == "i8":
+                    assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+                elif kind == "q4":
+                    assert mil.nnopt_register_q4_weight(wb, sb, N, K)
+                pool.append((wb, sb))
+            xb = x_i if K == INTER else x_h
+            yb = mil.Buffer(N * 2)
+            arr = mil.make_calls([(1, N, K, xb, pool[i % npool][0], yb) for i in range(max(npool, 32))])
+            mil.linear_batch(queue, arr)
+            ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 5) / len(arr)
+            with mil.Graph(queue) as g:
+                mil.linear_batch(queue, arr)
+            g.launch()
+            ms_g = time_region(mil, queue, g.launch, 5) / len(arr)
+            ms = min(ms, ms_g)
+            for wb, _ in pool:
+                mil.nnopt_unregister_weight(wb)
+            return {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                    "frac_hbm": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "bytes": nbytes}
+
+        detail["c1_fp16_gemv_1536x576"] = cold_gemv("f16", 1536, 576, 340)
+        detail["c2_int8_gemv_4864x896"] = cold_gemv("i8", INTER, H, 140)
+        detail["c2_int8_gemv_896x4864"] = cold_gemv("i8", H, INTER, 140)
+        detail["c3_q4_gemv_151936x896"] = cold_gemv("q4", VOCAB, H, 4)
+        detail["c3_int8_gemv_151936x896"] = {"us": roofline["us_per_launch"], "GBps": roofline["achieved"],
+                                             "frac_hbm": roofline["frac"], "bytes": lm_bytes}
+
+    # ---- CPU baseline: the oracle on a bounded sample of the same sweep -------------------
+    cpu = None
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        import oracle_lib as O
+        threads = O.lib.orc_max_threads()
+        xh = mil.synth_normal_f16(1, 1.0, (H,))
+        xi = mil.synth_normal_f16(2, 1.0, (INTER,))
+        sample_bytes, t0, reps = 0, time.time(), 0
+        while time.time() - t0 < 12.0 or reps < 2:
+            for name, N, K in LAYER_SHAPES:                    # layer 0 of the sweep ...
+                q, s = host_layer0[name]
+                O.gemv_i8(xi if K == INTER else xh, q, s.view(np.uint16), threads)
+                sample_bytes += N * K + 2 * N
+            O.gemv_i8(xh, lm_host[0], lm_host[1].view(np.uint16), threads)   # ... and the lm_head
+            sample_bytes += VOCAB * H + 2 * VOCAB
+            reps += 1
+        dt = time.time() - t0
+        cpu = {"value": round(sample_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+               "sample": f"{reps} x (layer 0's 7 int8 GEMVs + the lm_head GEMV), {sample_bytes} algorithmic "
+                         f"bytes in {dt:.1f} s, OpenMP over rows"}
+
+    out = {
+        "metric": "quant GEMV achieved HBM GB/s (% of peak) + us/decode-step, Qwen2.5-0.5B shapes",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 weights, fp16 activations, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "Qwen2.5-0.5B decode-step matmul sweep, batch 1, per-row int8: 24 x "
+                               "{q,k,v,o,gate,up,down} + lm_head = 169 GEMVs, 494873344 algorithmic bytes",
+                   "launch": launch_mode, "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+                   "us_per_decode_step": round(ms_step * 1e3, 1)},
+        "roofline": roofline, "cpu_baseline": cpu, "detail": detail,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

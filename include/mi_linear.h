@@ -1,0 +1,161 @@
+/*
+ * mi_linear.h -- C ABI of the MI355X (gfx950) weight-only quantized matmul path.
+ *
+ * Drop-in boundary for the `pytorch_linear` family of a8nova/adreno-llms: the
+ * entry points below are what a foreign-function binding for the projection /
+ * lm_head calls in src/models/<model>/src would bind.  Device pointers stand where the
+ * reference passes cl_mem handles, a stream (hipStream_t passed as void*, NULL =
+ * the default stream) stands where it passes a cl_command_queue.
+ *
+ * Conventions, as in the reference (QW/src/utils.h:98-121, QW/src/debug_utils.h:56-64):
+ *   - functions that the reference declares `bool` return 1 (work enqueued) or 0
+ *     (nothing usable was enqueued); every failure prints
+ *     "ERROR: <message> (<file>:<line>)" on stderr; no exceptions, no errno;
+ *   - calls are asynchronous: they return after the launch; work on one stream runs
+ *     in order, so `out` is visible to the next call on the same stream;
+ *   - x, W, scale and out are caller-owned; the library keeps only the registry
+ *     entries made by mi_register_*_weight, keyed by the raw pointer value;
+ *   - the quantisation of W is not an argument: it is looked up from the W pointer
+ *     (LF/src/utils.cpp:1286-1325: Q4 first, then int8, then fp16);
+ *   - layouts are the ones of the reference bundles (scripts/convert_hf_to_bin.py,
+ *     LF/scripts/quantize_weights.py, LF/scripts/quantize_q4.py): W [N,K] row-major,
+ *     fp16, or int8 with fp16 scale[N], or Q4 packed [N,K/2] (low nibble = even
+ *     element, value = nibble-8) with fp16 scale[N,K/32].
+ *
+ * Paths: QW/ = src/models/qwen2-5-0-5b/, LF/ = src/models/lfm2-5-350m/,
+ * SM/ = src/models/smollm2-135m-instruct/, LV/ = src/models/lfm2-5-vl-450m/.
+ */
+#ifndef MI_LINEAR_H
+#define MI_LINEAR_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- runtime plumbing: what the reference host code takes from cl.h ------------- */
+
+/* Select the GPU and check that it is a gfx950 part.  Replaces
+ * OpenCLContext::initialize (QW/src/opencl_context.cpp:171-205).  Returns 1/0. */
+int mi_init(int device);
+/* Name of the device's architecture ("gfx950..."), valid after mi_init. */
+const char* mi_device_arch(void);
+/* Number of compute units of the selected device. */
+int mi_device_cus(void);
+
+/* clCreateBuffer / clReleaseMemObject (QW/src/weights.cpp:262-293). */
+void* mi_malloc(size_t bytes);
+int   mi_free(void* dev_ptr);
+/* clEnqueueWriteBuffer / clEnqueueReadBuffer, blocking form. */
+int mi_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes, void* stream);
+int mi_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, void* stream);
+int mi_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
+int mi_memset(void* dst_dev, int byte, size_t bytes, void* stream);
+/* clCreateCommandQueue / clReleaseCommandQueue / clFinish (QW/src/opencl_context.cpp:196-205). */
+void* mi_stream_create(void);
+int   mi_stream_destroy(void* stream);
+int   mi_stream_sync(void* stream);
+/* Event timing on a stream; stands for CL_QUEUE_PROFILING_ENABLE + clGetEventProfilingInfo
+ * (QW/src/prof.cpp:34-135). */
+void* mi_event_create(void);
+int   mi_event_destroy(void* ev);
+int   mi_event_record(void* ev, void* stream);
+int   mi_event_sync(void* ev);
+float mi_event_elapsed_ms(void* start_ev, void* stop_ev);
+
+/* ---- weight registry ------------------------------------------------------------ */
+
+/* nnopt_register_int8_weight (LF/src/utils.h:129, LF/src/utils.cpp:357-368). */
+int mi_register_int8_weight(const void* W_int8, const void* scale_fp16, int N, int K);
+/* nnopt_register_q4_weight (LF/src/utils.h:134, LF/src/utils.cpp:584-595); K = unpacked K. */
+int mi_register_q4_weight(const void* W_q4, const void* scale_fp16, int N, int K);
+/* The reference never unregisters; provided so that a freed pointer can be reused. */
+int mi_unregister_weight(const void* W);
+/* 0 = not registered (fp16), 8 = int8, 4 = Q4. */
+int mi_weight_kind(const void* W);
+
+/* ---- the hot path --------------------------------------------------------------- */
+
+/* pytorch_linear (QW/src/utils.h:119-121, QW/src/utils.cpp:758-823, LF/src/utils.cpp:1263-1374):
+ * out[M,N] = x[M,K] @ W[N,K]^T, fp16 in/out, fp32 accumulate. */
+int mi_linear(void* stream, int M, int N, int K, const void* x, const void* W, void* out);
+
+/* pytorch_linear_add (QW/src/utils.h:133-135; int8 form SM/kernels/block_fused_int8.cl:105-174,
+ * 238-291): residual_inout[n] = fp16(f32(residual_inout[n]) + (W x)[n]).  M must be 1;
+ * returns 0 (caller runs the unfused path) otherwise. */
+int mi_linear_add(void* stream, int M, int N, int K, const void* x, const void* W, void* residual_inout);
+
+/* fused_gate_up_silu_m1 (QW/src/utils.h:157-159; SM/kernels/block_fused_int8.cl:176-236,
+ * SM/kernels/block_fused.cl:473-526): out[c] = fp16(silu(Wg x)[c] * (Wu x)[c]).  Wg and Wu
+ * must be of the same kind (both fp16 or both int8); returns 0 otherwise. */
+int mi_linear_gate_up_silu(void* stream, int N, int K, const void* x, const void* Wg, const void* Wu, void* out);
+
+/* dequant_int8_weight_to_fp16 (LV/src/utils.cpp:594-634, LV/kernels/lfm2_ops.cl:731-743):
+ * w16[n,k] = fp16(f32(q[n,k]) * f32(scale[n])). */
+int mi_dequant_int8_to_fp16(void* stream, const void* W_int8, const void* scale_fp16, int N, int K, void* w16);
+/* Debug view of the Q4 unpack (UNPACK8_FROM_PIXEL, LF/kernels/gemv_m1_q4.cl:31-40):
+ * w8[n,k] = nibble(n,k) - 8 as int8. */
+int mi_unpack_q4_to_int8(void* stream, const void* W_q4, int N, int K, void* w8);
+
+/* One call of mi_linear, for mi_linear_batch. */
+typedef struct mi_linear_call {
+    int M, N, K;
+    const void* x;
+    const void* W;
+    void* out;
+} mi_linear_call;
+
+/* Enqueues calls[0..n) in order on one stream, exactly as n calls of mi_linear would: the
+ * host-side loop of a decode step (Model::forward_chained_enqueue, QW/src/model.cpp:709-856,
+ * issues its ~170 projections this way).  Returns the number of calls enqueued (n on success). */
+int mi_linear_batch(void* stream, const mi_linear_call* calls, int n);
+
+/* Record / replay of everything enqueued on a stream between begin and end, as a HIP graph;
+ * the counterpart of the reference's recordable-queue replay of the decode step
+ * (NNOPT_RECORD, QW/src/model.cpp:709-720).  Only kernel launches may be recorded: no
+ * mi_malloc, mi_memcpy_* or mi_memset between begin and end. */
+int   mi_graph_begin(void* stream);
+void* mi_graph_end(void* stream);              /* returns an executable graph or NULL */
+int   mi_graph_launch(void* graph, void* stream);
+int   mi_graph_destroy(void* graph);
+
+/* Selects how M > 1 is computed for a quantised W: 0 (default) = MFMA GEMM with fused
+ * dequant for M >= 16 and batched GEMV below; 1 = always the batched GEMV, whose rows
+ * are bit-identical to M = 1 calls (the reference's prefill loop, LF/src/model.cpp:243-250). */
+void mi_set_gemm_mode(int mode);
+
+/* ---- offline tools (host) -------------------------------------------------------- */
+
+/* quantize_row_symmetric over N rows (LF/scripts/quantize_weights.py:53-57). */
+int mi_quantize_int8(const uint16_t* w_fp16, int N, int K, int8_t* q, uint16_t* scale_fp16);
+/* quantize_row_q4 over N rows (LF/scripts/quantize_q4.py:62-82); 0 if K % 32 != 0. */
+int mi_quantize_q4(const uint16_t* w_fp16, int N, int K, uint8_t* packed, uint16_t* scale_fp16);
+/* Host fp16 codec (QW/src/utils.cpp:497-564). */
+float    mi_f16_to_f32(uint16_t h);
+uint16_t mi_f32_to_f16(float f);
+/* Seeded synthetic tensors: n values ~ N(0, sigma) rounded to fp16.  Counter-based
+ * (splitmix64 of seed and index, Box-Muller in double), so any slice can be made
+ * independently and the bits do not depend on thread count. */
+void mi_synth_normal_f16(uint64_t seed, double sigma, size_t n, uint16_t* out);
+
+/* ---- weight bundles (.bin + .meta.json) ------------------------------------------ */
+
+/* Weights::load / parse_meta_json / get_buffer (QW/src/weights.cpp:22-140, 165-254, 262-293;
+ * int8 / q4_packed sizes LF/src/weights.cpp:143-148).  The .bin is mmap-ed. */
+void* mi_bundle_open(const char* bin_path, const char* meta_path);
+void  mi_bundle_close(void* bundle);
+int   mi_bundle_count(void* bundle);
+const char* mi_bundle_name(void* bundle, int index);              /* sorted-name order */
+/* Returns 1 and fills the outputs if the tensor exists.  dtype: "float16" | "int8" | "q4_packed". */
+int   mi_bundle_tensor(void* bundle, const char* name, const void** host_ptr, size_t* size_bytes,
+                       const char** dtype, int* ndim, int64_t shape[4]);
+/* Uploads every tensor to the device and registers each int8 / q4_packed tensor that has a
+ * "<name>.scale" (or "<name>.scales") sibling, as LF/src/main.cpp:527-566 does. Returns the
+ * number of registered weights, or -1 on error. */
+int   mi_bundle_upload(void* bundle);
+void* mi_bundle_device_ptr(void* bundle, const char* name);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
