@@ -41,7 +41,14 @@ __device__ __forceinline__ float hi_f(uint32_t p) {
     return __half2float(__ushort_as_half(static_cast<unsigned short>(p >> 16)));
 }
 __device__ __forceinline__ float h_f(uint16_t h) { return __half2float(__ushort_as_half(h)); }
-__device__ __forceinline__ uint16_t f_h(float f) { return __half_as_ushort(__float2half_rn(f)); }
+// fp32 -> fp16, round to nearest even.  The empty asm pins the fp32 value in a register
+// first: without it the compiler folds a preceding multiply or fma into v_fma_mixlo_f16,
+// which rounds once to fp16, while the reference rounds the product to fp32 and then
+// stores it as half (two roundings; they differ on about one value in 8000).
+__device__ __forceinline__ uint16_t f_h(float f) {
+    asm volatile("" : "+v"(f));
+    return __half_as_ushort(__float2half_rn(f));
+}
 
 // Two nibbles (bits 0-3 and 16-19 of v) -> two fp16 values (nibble - 8), exact:
 // 0x6400 | n is the half 1024 + n, and (1024 + n) - 1032 is exact.
