@@ -43,7 +43,10 @@ struct GemvCall {
 };
 
 // gemv.hip
+constexpr int kMaxSegments = 4;
 bool launch_gemv(hipStream_t s, const GemvCall& c);
+// n <= kMaxSegments calls that share x, K, M, weight kind and epilogue, as one launch.
+bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n);
 bool launch_gate_up_silu(hipStream_t s, WeightKind kind, int N, int K, const void* x,
                          const void* Wg, const void* sg, const void* Wu, const void* su, void* out);
 bool launch_dequant_int8(hipStream_t s, const void* q, const void* scale, int N, int K, void* w16);

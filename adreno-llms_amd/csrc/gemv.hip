@@ -10,15 +10,22 @@
 // the 64 accumulators of a row are "virtual lanes", and one hardware lane owns VL
 // consecutive virtual lanes.  With VL = 4 a lane reads 16 bytes of int8/Q4 weights per
 // iteration (one global_load_dwordx4), 16 lanes cover a row-iteration and a 64-wide
-// wavefront works on 4 rows at once; VL = 2 and VL = 1 trade load width for more
-// wavefronts when N is small.  Tree steps with s >= VL are cross-lane adds inside the
-// 64/VL-lane group, steps with s < VL are adds between a lane's own accumulators.
+// wavefront works on 4 rows at once ("a row batch"); VL = 2 and VL = 1 trade load width
+// for more wavefronts when N is small.  Tree steps with s >= VL are cross-lane adds inside
+// the 64/VL-lane group (DPP row shifts), steps with s < VL are adds between a lane's own
+// accumulators.
 //
 // A lane's K positions do not depend on the row, so in the fixed-K kernels the lane loads
-// its slice of x once into registers and then streams rows: the inner loop issues only
-// weight loads (every byte of W is read exactly once, fully coalesced) and two VALU
-// operations per int8 weight (v_cvt_f32_i32 with a byte select, v_fma_mix_f32 taking x
-// straight from its fp16 register half).  No MFMA: at batch 1 the op is HBM-bound.
+// its slice of x once into registers and then streams row batches: every byte of W is
+// read exactly once, fully coalesced, with non-temporal loads, and while one batch is
+// being multiplied the next one is already in flight (two register buffers, the loop is
+// unrolled by two so no buffer is ever copied).  Per int8 weight the inner loop is two
+// VALU operations (v_cvt_f32_i32 with a byte select, v_fma_mix_f32 / v_fma_f32).  No MFMA:
+// at batch 1 the op is HBM-bound.
+//
+// Several GEMVs that read the same x and have the same K and weight kind (q/k/v, gate/up)
+// can be given to one launch as "segments": the row batches of all segments form one
+// index space.
 #include "common.h"
 #include <hip/hip_fp16.h>
 
@@ -29,10 +36,26 @@ constexpr int kWave = 64;
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = kWave * kWavesPerBlock;
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
 template <int KIND> struct WT;
 template <> struct WT<WK_F16> { static constexpr int EPV = 4, BPV = 8; };  // elements / bytes per virtual lane
 template <> struct WT<WK_I8>  { static constexpr int EPV = 4, BPV = 4; };
 template <> struct WT<WK_Q4>  { static constexpr int EPV = 8, BPV = 4; };
+
+struct Seg {
+    const uint8_t*  W;
+    const uint16_t* sc;
+    uint16_t*       y;
+    int N;
+    int first;       // index of the segment's first row batch in the launch
+};
+struct SegList {
+    Seg s[kMaxSegments];
+    int nseg;
+    int nbatch;      // row batches of all segments
+};
 
 __device__ __forceinline__ float lo_f(uint32_t p) {
     return __half2float(__ushort_as_half(static_cast<unsigned short>(p & 0xffffu)));
@@ -41,6 +64,7 @@ __device__ __forceinline__ float hi_f(uint32_t p) {
     return __half2float(__ushort_as_half(static_cast<unsigned short>(p >> 16)));
 }
 __device__ __forceinline__ float h_f(uint16_t h) { return __half2float(__ushort_as_half(h)); }
+
 // fp32 -> fp16, round to nearest even.  The empty asm pins the fp32 value in a register
 // first: without it the compiler folds a preceding multiply or fma into v_fma_mixlo_f16,
 // which rounds once to fp16, while the reference rounds the product to fp32 and then
@@ -95,30 +119,50 @@ __device__ __forceinline__ float vlane_step(float acc, const uint32_t* w, const 
     }
 }
 
-template <int ND> __device__ __forceinline__ void load_dwords(uint32_t* dst, const void* src) {
+// ND dwords from 4*ND-byte aligned memory; NT = non-temporal (weights are used once).
+template <int ND, bool NT> __device__ __forceinline__ void load_dwords(uint32_t* dst, const void* src) {
     if constexpr (ND == 1) {
-        dst[0] = *static_cast<const uint32_t*>(src);
+        dst[0] = NT ? __builtin_nontemporal_load(static_cast<const uint32_t*>(src))
+                    : *static_cast<const uint32_t*>(src);
     } else if constexpr (ND == 2) {
-        const uint2 v = *static_cast<const uint2*>(src);
+        const u32x2 v = NT ? __builtin_nontemporal_load(static_cast<const u32x2*>(src))
+                           : *static_cast<const u32x2*>(src);
         dst[0] = v.x; dst[1] = v.y;
     } else {
         static_assert(ND % 4 == 0, "dword count");
         #pragma unroll
         for (int i = 0; i < ND / 4; ++i) {
-            const uint4 v = static_cast<const uint4*>(src)[i];
+            const u32x4 v = NT ? __builtin_nontemporal_load(static_cast<const u32x4*>(src) + i)
+                               : static_cast<const u32x4*>(src)[i];
             dst[4 * i] = v.x; dst[4 * i + 1] = v.y; dst[4 * i + 2] = v.z; dst[4 * i + 3] = v.w;
         }
     }
 }
 
-// The 64-virtual-lane tree of the reference, on VL accumulators per lane.
+// a + (value of lane i+SH), inside a row of 16 lanes: DPP row_shl.  Lanes whose source
+// falls outside the row add 0; they are lanes whose result the tree never uses.
+template <int SH> __device__ __forceinline__ float add_from_above(float a) {
+    const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(a), 0x100 + SH, 0xf, 0xf, true);
+    return a + __int_as_float(t);
+}
+
+// The 64-virtual-lane tree of the reference, on VL accumulators per lane: steps
+// s = 32 .. VL pair lane g with lane g + s/VL, steps s < VL pair a lane's own accumulators.
 template <int VL> __device__ __forceinline__ float reduce_row(float (&acc)[VL]) {
     constexpr int LPR = kWave / VL;
     #pragma unroll
-    for (int off = LPR / 2; off >= 1; off >>= 1) {
-        #pragma unroll
-        for (int v = 0; v < VL; ++v) acc[v] = acc[v] + __shfl_down(acc[v], off, LPR);
+    for (int v = 0; v < VL; ++v) {
+        if constexpr (LPR >= 64) acc[v] = acc[v] + __shfl_down(acc[v], 32, 64);
+        if constexpr (LPR >= 32) acc[v] = acc[v] + __shfl_down(acc[v], 16, LPR);
     }
+    #pragma unroll
+    for (int v = 0; v < VL; ++v) acc[v] = add_from_above<8>(acc[v]);
+    #pragma unroll
+    for (int v = 0; v < VL; ++v) acc[v] = add_from_above<4>(acc[v]);
+    #pragma unroll
+    for (int v = 0; v < VL; ++v) acc[v] = add_from_above<2>(acc[v]);
+    #pragma unroll
+    for (int v = 0; v < VL; ++v) acc[v] = add_from_above<1>(acc[v]);
     #pragma unroll
     for (int s = VL / 2; s >= 1; s >>= 1) {
         #pragma unroll
@@ -127,24 +171,24 @@ template <int VL> __device__ __forceinline__ float reduce_row(float (&acc)[VL]) 
     return acc[0];
 }
 
-template <int KIND, int EPI>
-__device__ __forceinline__ void epilogue(float sum, const uint16_t* sc, uint16_t* y, int row) {
-    if constexpr (KIND == WK_I8) {
-        const float s = h_f(sc[row]);
-        if constexpr (EPI == EPI_ADD) y[row] = f_h(fmaf(sum, s, h_f(y[row])));
-        else y[row] = f_h(sum * s);
-    } else {
-        if constexpr (EPI == EPI_ADD) y[row] = f_h(sum + h_f(y[row]));
-        else y[row] = f_h(sum);
-    }
+// Segment that holds row batch rb.  rb must be uniform over the wavefront (it is built
+// from readfirstlane values), so the selects below are scalar and the segment table is
+// read through the scalar cache: a vector load here would make every fetch wait for all
+// outstanding weight loads.
+__device__ __forceinline__ Seg find_segment(const SegList& L, int rb) {
+    Seg sg = L.s[0];
+    #pragma unroll
+    for (int i = 1; i < kMaxSegments; ++i)
+        if (i < L.nseg && rb >= L.s[i].first) sg = L.s[i];
+    return sg;
 }
 
 // ---- K known at compile time: x lives in registers ---------------------------------
-template <int KIND, int KT, int VL, int EPI>
-__global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restrict__ x,
-                                                       const uint8_t* __restrict__ W,
-                                                       const uint16_t* __restrict__ sc,
-                                                       uint16_t* __restrict__ y, int N) {
+//
+// PIPE: each wavefront walks several row batches and keeps the next one in flight while it
+// multiplies the current one.  Without PIPE a wavefront is expected to own one batch.
+template <int KIND, int KT, int VL, int EPI, bool PIPE>
+__global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restrict__ x, const SegList L) {
     using T = WT<KIND>;
     constexpr int LPR = kWave / VL, RPW = VL;
     constexpr int EIT = kWave * T::EPV;                 // elements per K-iteration
@@ -154,62 +198,107 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     constexpr int ROWB = KT / T::EPV * T::BPV;          // bytes per weight row
     constexpr int ITB = kWave * T::BPV;                 // weight bytes per row and iteration
 
-    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int g = lane % LPR, r = lane / LPR;
     const int koff = g * VL * T::EPV;
-    x += static_cast<size_t>(blockIdx.y) * KT;
-    y += static_cast<size_t>(blockIdx.y) * N;
+    const int m = blockIdx.y;
+    x += static_cast<size_t>(m) * KT;
 
     uint32_t xr[NIT][XD];
     #pragma unroll
     for (int j = 0; j < NIT; ++j) {
-        if (j * EIT + koff < KT) load_dwords<XD>(xr[j], x + j * EIT + koff);
+        if (j * EIT + koff < KT) load_dwords<XD, false>(xr[j], x + j * EIT + koff);
         else {
             #pragma unroll
             for (int i = 0; i < XD; ++i) xr[j][i] = 0u;
         }
     }
 
-    const int nbatch = (N + RPW - 1) / RPW;
-    for (int rb = blockIdx.x * kWavesPerBlock + wave; rb < nbatch; rb += gridDim.x * kWavesPerBlock) {
-        const int row = rb * RPW + r;
-        const bool valid = row < N;
-        const int rowc = valid ? row : N - 1;
-        const uint8_t* wrow = W + static_cast<size_t>(rowc) * ROWB + koff / T::EPV * T::BPV;
-
-        uint32_t wr[NIT][WD];
-        float sf[NIT];
+    // One row batch in registers: weights, scales and (EPI_ADD) the residual, all fetched
+    // together so that the epilogue never waits on a late load.
+    struct Batch {
+        uint32_t w[NIT][WD];
+        uint16_t s[KIND == WK_Q4 ? NIT : 1];
+        uint16_t res;
+        uint16_t* yrow;     // null when the lane's row is past N
+    };
+    auto fetch = [&](Batch& b, int rb) {
+        const Seg sg = find_segment(L, rb);
+        const int row = (rb - sg.first) * RPW + r;
+        const bool valid = row < sg.N;
+        const int rowc = valid ? row : sg.N - 1;
+        uint16_t* yp = sg.y + static_cast<size_t>(m) * sg.N + rowc;
+        b.yrow = valid ? yp : nullptr;
+        if constexpr (KIND == WK_I8) b.s[0] = sg.sc[rowc];
+        if constexpr (EPI == EPI_ADD) b.res = *yp;
+        const uint8_t* wrow = sg.W + static_cast<size_t>(rowc) * ROWB;
+        const int lane_off = koff / T::EPV * T::BPV;
         #pragma unroll
         for (int j = 0; j < NIT; ++j) {
-            if (j * EIT + koff < KT) {
-                load_dwords<WD>(wr[j], wrow + j * ITB);
-                if constexpr (KIND == WK_Q4)
-                    sf[j] = h_f(sc[static_cast<size_t>(rowc) * (KT / 32) + j * 16 + (g * VL) / 4]);
-                else sf[j] = 0.0f;
-            }
+            // lanes idle in a partial last iteration re-read the start of the row, so that
+            // every lane issues the same number of loads (the value is never used)
+            const bool active = j * EIT + koff < KT;
+            load_dwords<WD, true>(b.w[j], wrow + (active ? j * ITB + lane_off : 0));
+            if constexpr (KIND == WK_Q4)
+                b.s[j] = sg.sc[static_cast<size_t>(rowc) * (KT / 32) + (active ? j * 16 + (g * VL) / 4 : 0)];
         }
+    };
+    auto consume = [&](const Batch& b) {
         float acc[VL];
         #pragma unroll
         for (int v = 0; v < VL; ++v) acc[v] = 0.0f;
         #pragma unroll
         for (int j = 0; j < NIT; ++j) {
             if (j * EIT + koff < KT) {
+                const float sf = KIND == WK_Q4 ? h_f(b.s[KIND == WK_Q4 ? j : 0]) : 0.0f;
                 #pragma unroll
                 for (int v = 0; v < VL; ++v)
-                    acc[v] = vlane_step<KIND>(acc[v], &wr[j][v * T::BPV / 4], &xr[j][v * T::EPV / 2], sf[j]);
+                    acc[v] = vlane_step<KIND>(acc[v], &b.w[j][v * T::BPV / 4], &xr[j][v * T::EPV / 2], sf);
             }
         }
         const float sum = reduce_row<VL>(acc);
-        if (g == 0 && valid) epilogue<KIND, EPI>(sum, sc, y, row);
+        if (g == 0 && b.yrow) {
+            float out;
+            if constexpr (KIND == WK_I8) {
+                const float s = h_f(b.s[0]);
+                out = EPI == EPI_ADD ? fmaf(sum, s, h_f(b.res)) : sum * s;
+            } else {
+                out = EPI == EPI_ADD ? sum + h_f(b.res) : sum;
+            }
+            *b.yrow = f_h(out);
+        }
+    };
+
+    const int nw = gridDim.x * kWavesPerBlock;
+    int rb = blockIdx.x * kWavesPerBlock + wave;
+    if (rb >= L.nbatch) return;
+    if constexpr (!PIPE) {
+        for (; rb < L.nbatch; rb += nw) {
+            Batch b;
+            fetch(b, rb);
+            consume(b);
+        }
+    } else {
+        Batch b0, b1;
+        fetch(b0, rb);
+        while (true) {
+            // the prefetch of a batch past the end re-reads the current one (cached, unused)
+            fetch(b1, rb + nw < L.nbatch ? rb + nw : rb);
+            consume(b0);
+            rb += nw;
+            if (rb >= L.nbatch) break;
+            fetch(b0, rb + nw < L.nbatch ? rb + nw : rb);
+            consume(b1);
+            rb += nw;
+            if (rb >= L.nbatch) break;
+        }
     }
 }
 
 // ---- K known at run time: x is staged once per block in LDS ------------------------
 template <int KIND, int VL, int EPI>
-__global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict__ x,
-                                                     const uint8_t* __restrict__ W,
-                                                     const uint16_t* __restrict__ sc,
-                                                     uint16_t* __restrict__ y, int N, int K) {
+__global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict__ x, const SegList L, int K) {
     using T = WT<KIND>;
     constexpr int LPR = kWave / VL, RPW = VL;
     constexpr int EIT = kWave * T::EPV;
@@ -218,24 +307,25 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict_
     constexpr int ITB = kWave * T::BPV;
     extern __shared__ uint32_t xs[];                    // K/2 dwords of packed fp16
 
-    x += static_cast<size_t>(blockIdx.y) * K;
-    y += static_cast<size_t>(blockIdx.y) * N;
+    const int m = blockIdx.y;
+    x += static_cast<size_t>(m) * K;
     for (int i = threadIdx.x; i < K / 2; i += kBlock) xs[i] = reinterpret_cast<const uint32_t*>(x)[i];
     __syncthreads();
 
-    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int g = lane % LPR, r = lane / LPR;
     const int koff = g * VL * T::EPV;
     const size_t rowb = static_cast<size_t>(K) / T::EPV * T::BPV;
     const int nit = (K + EIT - 1) / EIT;
-    const int nbatch = (N + RPW - 1) / RPW;
 
-    for (int rb = blockIdx.x * kWavesPerBlock + wave; rb < nbatch; rb += gridDim.x * kWavesPerBlock) {
-        const int row = rb * RPW + r;
-        const bool valid = row < N;
-        const int rowc = valid ? row : N - 1;
-        const uint8_t* wrow = W + static_cast<size_t>(rowc) * rowb + koff / T::EPV * T::BPV;
-        const uint16_t* srow = sc + static_cast<size_t>(rowc) * (K / 32) + (g * VL) / 4;
+    for (int rb = blockIdx.x * kWavesPerBlock + wave; rb < L.nbatch; rb += gridDim.x * kWavesPerBlock) {
+        const Seg sg = find_segment(L, rb);
+        const int row = (rb - sg.first) * RPW + r;
+        const bool valid = row < sg.N;
+        const int rowc = valid ? row : sg.N - 1;
+        const uint8_t* wrow = sg.W + static_cast<size_t>(rowc) * rowb + koff / T::EPV * T::BPV;
+        const uint16_t* srow = sg.sc + static_cast<size_t>(rowc) * (K / 32) + (g * VL) / 4;
         float acc[VL];
         #pragma unroll
         for (int v = 0; v < VL; ++v) acc[v] = 0.0f;
@@ -244,7 +334,7 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict_
             const int k = j * EIT + koff;
             if (k < K) {
                 uint32_t wr[WD], xr[XD];
-                load_dwords<WD>(wr, wrow + static_cast<size_t>(j) * ITB);
+                load_dwords<WD, true>(wr, wrow + static_cast<size_t>(j) * ITB);
                 #pragma unroll
                 for (int i = 0; i < XD; ++i) xr[i] = xs[k / 2 + i];
                 float sf = 0.0f;
@@ -255,7 +345,17 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict_
             }
         }
         const float sum = reduce_row<VL>(acc);
-        if (g == 0 && valid) epilogue<KIND, EPI>(sum, sc, y, row);
+        if (g == 0 && valid) {
+            uint16_t* yp = sg.y + static_cast<size_t>(m) * sg.N + row;
+            float out;
+            if constexpr (KIND == WK_I8) {
+                const float s = h_f(sg.sc[row]);
+                out = EPI == EPI_ADD ? fmaf(sum, s, h_f(*yp)) : sum * s;
+            } else {
+                out = EPI == EPI_ADD ? sum + h_f(*yp) : sum;
+            }
+            *yp = f_h(out);
+        }
     }
 }
 
@@ -299,7 +399,8 @@ __global__ __launch_bounds__(kBlock) void gate_up_silu_any_k(const uint16_t* __r
     for (int i = threadIdx.x; i < K / 2; i += kBlock) xs[i] = reinterpret_cast<const uint32_t*>(x)[i];
     __syncthreads();
 
-    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int g = lane % LPR, r = lane / LPR;
     const int koff = g * VL * T::EPV;
     const size_t rowb = static_cast<size_t>(K) / T::EPV * T::BPV;
@@ -319,8 +420,8 @@ __global__ __launch_bounds__(kBlock) void gate_up_silu_any_k(const uint16_t* __r
             const int k = j * EIT + koff;
             if (k < K) {
                 uint32_t wg[WD], wu[WD], xr[XD];
-                load_dwords<WD>(wg, Wg + off + static_cast<size_t>(j) * ITB);
-                load_dwords<WD>(wu, Wu + off + static_cast<size_t>(j) * ITB);
+                load_dwords<WD, true>(wg, Wg + off + static_cast<size_t>(j) * ITB);
+                load_dwords<WD, true>(wu, Wu + off + static_cast<size_t>(j) * ITB);
                 #pragma unroll
                 for (int i = 0; i < XD; ++i) xr[i] = xs[k / 2 + i];
                 #pragma unroll
@@ -361,10 +462,14 @@ __global__ __launch_bounds__(256) void unpack_q4_kernel(const uint8_t* __restric
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
+// Wavefronts that one launch keeps resident when it streams many row batches: 3 blocks of
+// 4 wavefronts per CU (measured best for the pipelined kernels on MI355X).
+inline int resident_waves() { return device_info().cus * 3 * kWavesPerBlock; }
+
 // Widest lane tile that still gives every SIMD of the chip a wavefront; when no tile
 // reaches that, the narrowest one (most wavefronts).  A tile of VL fits when a lane's
 // VL virtual lanes are whole in the K tail.
-int pick_vl(WeightKind kind, int M, int N, int K) {
+int pick_vl(WeightKind kind, int M, long rows, int K) {
     const int epv = kind == WK_Q4 ? 8 : 4;
     const int max_vl = kind == WK_F16 ? 2 : 4;
     const long waves_wanted = 4L * device_info().cus;
@@ -372,40 +477,61 @@ int pick_vl(WeightKind kind, int M, int N, int K) {
     for (int vl = max_vl; vl >= 1; vl >>= 1) {
         if (K % (vl * epv) != 0) continue;
         narrowest = vl;
-        if (static_cast<long>(M) * ((N + vl - 1) / vl) >= waves_wanted) return vl;
+        if (static_cast<long>(M) * ((rows + vl - 1) / vl) >= waves_wanted) return vl;
     }
     return narrowest;
 }
 
-dim3 grid_for(int M, int N, int vl) {
-    const int nbatch = (N + vl - 1) / vl;
-    const int blocks = (nbatch + kWavesPerBlock - 1) / kWavesPerBlock;
-    const int cap = device_info().cus * 8;                  // 32 wavefronts per CU
-    return dim3(blocks < cap ? blocks : cap, M, 1);
+struct Plan {
+    SegList L;
+    dim3 grid;
+    bool pipe;
+};
+
+Plan make_plan(const GemvCall* calls, int n, int vl) {
+    Plan p{};
+    int first = 0;
+    for (int i = 0; i < n; ++i) {
+        p.L.s[i] = Seg{static_cast<const uint8_t*>(calls[i].W), static_cast<const uint16_t*>(calls[i].scale),
+                       static_cast<uint16_t*>(calls[i].y), calls[i].N, first};
+        first += (calls[i].N + vl - 1) / vl;
+    }
+    p.L.nseg = n;
+    p.L.nbatch = first;
+    const int cap = resident_waves();
+    int waves = first;
+    p.pipe = false;
+    if (first > cap) {
+        // several batches per wavefront, the same number for all of them (+-1)
+        const int per_wave = (first + cap - 1) / cap;
+        waves = (first + per_wave - 1) / per_wave;
+        p.pipe = true;
+    }
+    p.grid = dim3((waves + kWavesPerBlock - 1) / kWavesPerBlock, calls[0].M, 1);
+    return p;
 }
 
 template <int KIND, int VL, int EPI>
-bool launch_kind_vl(hipStream_t s, const GemvCall& c) {
-    const auto* x = static_cast<const uint16_t*>(c.x);
-    const auto* W = static_cast<const uint8_t*>(c.W);
-    const auto* sc = static_cast<const uint16_t*>(c.scale);
-    auto* y = static_cast<uint16_t*>(c.y);
-    const dim3 grid = grid_for(c.M, c.N, VL);
-#define MI_FIXED(KT)                                                                          \
-    case KT:                                                                                  \
-        hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI>), grid, dim3(kBlock), 0, s, x, W, \
-                           sc, y, c.N);                                                       \
+bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
+    const Plan p = make_plan(calls, n, VL);
+    const auto* x = static_cast<const uint16_t*>(calls[0].x);
+    const int K = calls[0].K;
+#define MI_FIXED(KT, PIPE_OK)                                                                            \
+    case KT:                                                                                             \
+        if (PIPE_OK && p.pipe)                                                                           \
+            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, PIPE_OK>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+        else                                                                                             \
+            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, false>), p.grid, dim3(kBlock), 0, s, x, p.L);  \
         break;
-    switch (c.K) {
-        MI_FIXED(576)
-        MI_FIXED(896)
-        MI_FIXED(1024)
-        MI_FIXED(1536)
-        MI_FIXED(4864)
+    switch (K) {
+        MI_FIXED(576, true)
+        MI_FIXED(896, true)
+        MI_FIXED(1024, true)
+        MI_FIXED(1536, true)
+        MI_FIXED(4864, false)
         default: {
-            const size_t lds = static_cast<size_t>(c.K) * 2;
-            hipLaunchKernelGGL((gemv_any_k<KIND, VL, EPI>), grid, dim3(kBlock), lds, s, x, W, sc, y,
-                               c.N, c.K);
+            const size_t lds = static_cast<size_t>(K) * 2;
+            hipLaunchKernelGGL((gemv_any_k<KIND, VL, EPI>), p.grid, dim3(kBlock), lds, s, x, p.L, K);
         }
     }
 #undef MI_FIXED
@@ -413,17 +539,15 @@ bool launch_kind_vl(hipStream_t s, const GemvCall& c) {
 }
 
 template <int KIND, int EPI>
-bool launch_kind(hipStream_t s, const GemvCall& c, int vl) {
+bool launch_kind(hipStream_t s, const GemvCall* calls, int n, int vl) {
     if constexpr (KIND != WK_F16) {
-        if (vl == 4) return launch_kind_vl<KIND, 4, EPI>(s, c);
+        if (vl == 4) return launch_kind_vl<KIND, 4, EPI>(s, calls, n);
     }
-    if (vl == 2) return launch_kind_vl<KIND, 2, EPI>(s, c);
-    return launch_kind_vl<KIND, 1, EPI>(s, c);
+    if (vl == 2) return launch_kind_vl<KIND, 2, EPI>(s, calls, n);
+    return launch_kind_vl<KIND, 1, EPI>(s, calls, n);
 }
 
-}  // namespace
-
-bool launch_gemv(hipStream_t s, const GemvCall& c) {
+bool check_call(const GemvCall& c) {
     const int epv = c.kind == WK_Q4 ? 32 : 4;               // Q4 needs whole scale blocks
     if (c.M < 1 || c.N < 1 || c.K < 1 || c.K % epv != 0) {
         MI_ERROR_FMT("gemv: unsupported shape M=%d N=%d K=%d (K must be a multiple of %d)", c.M, c.N,
@@ -440,15 +564,38 @@ bool launch_gemv(hipStream_t s, const GemvCall& c) {
         MI_ERROR_FMT("gemv: null or misaligned operand (x and W need 16-byte alignment)");
         return false;
     }
-    const int vl = pick_vl(c.kind, c.M, c.N, c.K);
+    return true;
+}
+
+}  // namespace
+
+bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
+    if (n < 1 || n > kMaxSegments) {
+        MI_ERROR_FMT("gemv: %d segments in one launch (1..%d allowed)", n, kMaxSegments);
+        return false;
+    }
+    long rows = 0;
+    for (int i = 0; i < n; ++i) {
+        if (!check_call(calls[i])) return false;
+        if (calls[i].x != calls[0].x || calls[i].K != calls[0].K || calls[i].kind != calls[0].kind ||
+            calls[i].M != calls[0].M || calls[i].epi != calls[0].epi) {
+            MI_ERROR_FMT("gemv: segments of one launch must share x, K, M, weight kind and epilogue");
+            return false;
+        }
+        rows += calls[i].N;
+    }
+    const GemvCall& c = calls[0];
+    const int vl = pick_vl(c.kind, c.M, rows, c.K);
     const bool add = c.epi == EPI_ADD;
     switch (c.kind) {
-        case WK_F16: return add ? launch_kind<WK_F16, EPI_ADD>(s, c, vl) : launch_kind<WK_F16, EPI_STORE>(s, c, vl);
-        case WK_I8:  return add ? launch_kind<WK_I8, EPI_ADD>(s, c, vl) : launch_kind<WK_I8, EPI_STORE>(s, c, vl);
-        case WK_Q4:  return add ? launch_kind<WK_Q4, EPI_ADD>(s, c, vl) : launch_kind<WK_Q4, EPI_STORE>(s, c, vl);
+        case WK_F16: return add ? launch_kind<WK_F16, EPI_ADD>(s, calls, n, vl) : launch_kind<WK_F16, EPI_STORE>(s, calls, n, vl);
+        case WK_I8:  return add ? launch_kind<WK_I8, EPI_ADD>(s, calls, n, vl) : launch_kind<WK_I8, EPI_STORE>(s, calls, n, vl);
+        case WK_Q4:  return add ? launch_kind<WK_Q4, EPI_ADD>(s, calls, n, vl) : launch_kind<WK_Q4, EPI_STORE>(s, calls, n, vl);
     }
     return false;
 }
+
+bool launch_gemv(hipStream_t s, const GemvCall& c) { return launch_gemv_group(s, &c, 1); }
 
 bool launch_gate_up_silu(hipStream_t s, WeightKind kind, int N, int K, const void* x, const void* Wg,
                          const void* sg, const void* Wu, const void* su, void* out) {
@@ -461,7 +608,10 @@ bool launch_gate_up_silu(hipStream_t s, WeightKind kind, int N, int K, const voi
         return false;
     }
     const int vl = pick_vl(kind, 1, N, K);
-    const dim3 grid = grid_for(1, N, vl);
+    const int nbatch = (N + vl - 1) / vl;
+    const int cap = resident_waves();
+    const int waves = nbatch < cap ? nbatch : cap;
+    const dim3 grid((waves + kWavesPerBlock - 1) / kWavesPerBlock, 1, 1);
     const size_t lds = static_cast<size_t>(K) * 2;
     const auto* xp = static_cast<const uint16_t*>(x);
     const auto* g8 = static_cast<const uint8_t*>(Wg);

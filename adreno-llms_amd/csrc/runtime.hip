@@ -200,11 +200,58 @@ int mi_linear(void* stream, int M, int N, int K, const void* x, const void* W, v
     return launch_gemv(as_stream(stream), c) ? 1 : 0;
 }
 
+// True when [a, a+na) and [b, b+nb) share a byte.
+static bool overlaps(const void* a, size_t na, const void* b, size_t nb) {
+    const auto pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+    return pa < pb + nb && pb < pa + na;
+}
+
 int mi_linear_batch(void* stream, const mi_linear_call* calls, int n) {
+    if (!ensure_init()) return 0;
     if (!calls || n < 0) { MI_ERROR_FMT("mi_linear_batch: bad argument"); return 0; }
-    for (int i = 0; i < n; ++i) {
-        const mi_linear_call& c = calls[i];
-        if (!mi_linear(stream, c.M, c.N, c.K, c.x, c.W, c.out)) return i;
+    // Consecutive GEMV calls that read the same x with the same K and weight kind, and
+    // whose outputs touch neither that x nor each other, cannot observe one another: they
+    // go out as one launch (q/k/v and gate/up of a decode step do).  Everything else is
+    // enqueued call by call, in order.
+    int i = 0;
+    while (i < n) {
+        const mi_linear_call& c0 = calls[i];
+        Entry e0;
+        const bool groupable = c0.M >= 1 && c0.M < 16 && c0.N > 0 && c0.K > 0 && c0.x && c0.W && c0.out &&
+                               resolve("mi_linear_batch", c0.W, c0.N, c0.K, &e0);
+        if (!groupable) {
+            if (!mi_linear(stream, c0.M, c0.N, c0.K, c0.x, c0.W, c0.out)) return i;
+            ++i;
+            continue;
+        }
+        GemvCall group[kMaxSegments];
+        int g = 0;
+        const size_t xbytes = static_cast<size_t>(c0.M) * c0.K * 2;
+        while (i + g < n && g < kMaxSegments) {
+            const mi_linear_call& c = calls[i + g];
+            Entry e;
+            if (g > 0) {
+                if (c.x != c0.x || c.K != c0.K || c.M != c0.M || c.N <= 0 || !c.W || !c.out) break;
+                if (!lookup(c.W, &e)) e = Entry{WK_F16, nullptr, c.N, c.K};
+                if (e.kind != e0.kind || e.N != c.N || e.K != c.K) break;
+            } else e = e0;
+            const size_t obytes = static_cast<size_t>(c.M) * c.N * 2;
+            bool clash = overlaps(c.out, obytes, c0.x, xbytes);
+            for (int j = 0; j < g && !clash; ++j)
+                clash = overlaps(c.out, obytes, group[j].y, static_cast<size_t>(group[j].M) * group[j].N * 2);
+            if (clash) break;
+            GemvCall& d = group[g];
+            d.x = c.x; d.W = c.W; d.scale = e.scale; d.y = c.out;
+            d.M = c.M; d.N = c.N; d.K = c.K; d.kind = e.kind; d.epi = EPI_STORE;
+            ++g;
+        }
+        if (g == 0) {                                   // out aliases x: leave it to mi_linear
+            if (!mi_linear(stream, c0.M, c0.N, c0.K, c0.x, c0.W, c0.out)) return i;
+            ++i;
+            continue;
+        }
+        if (!launch_gemv_group(as_stream(stream), group, g)) return i;
+        i += g;
     }
     return n;
 }

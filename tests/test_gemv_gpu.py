@@ -264,6 +264,64 @@ def test_batch_and_graph_replay(queue):
         mil.nnopt_unregister_weight(b)
 
 
+@pytest.mark.parametrize("kind", ["i8", "q4", "f16"])
+def test_batch_merges_independent_calls_bit_exact(queue, kind):
+    """q/k/v-style calls (same x, different W and out) go out as one launch; the results must
+    equal separate calls, and calls that depend on each other must still run in order."""
+    K = 896
+    Ns = [896, 128, 128, 36, 4864]                  # five calls: more than one launch can hold
+    x = synth_x(40, K)
+    xb = mil.Buffer.from_host(x)
+    keep, calls, wants = [], [], []
+    for i, N in enumerate(Ns):
+        W = synth_w(41 + i, N, K)
+        ob = mil.Buffer.from_host(np.zeros(N, np.uint16))
+        if kind == "i8":
+            q, s = mil.quantize_int8(W)
+            Wb, sb = mil.Buffer.from_host(q), mil.Buffer.from_host(s)
+            assert mil.nnopt_register_int8_weight(Wb, sb, N, K)
+            wants.append(O.gemv_i8(x, q, s.view(np.uint16)))
+        elif kind == "q4":
+            p, sc = mil.quantize_q4(W)
+            Wb, sb = mil.Buffer.from_host(p), mil.Buffer.from_host(sc)
+            assert mil.nnopt_register_q4_weight(Wb, sb, N, K)
+            wants.append(O.gemv_q4(x, p, sc.view(np.uint16)))
+        else:
+            Wb, sb = mil.Buffer.from_host(W), None
+            wants.append(O.gemv_f16(x, W))
+        keep += [Wb, sb, ob]
+        calls.append((1, N, K, xb, Wb, ob))
+    arr = mil.make_calls(calls)
+    assert mil.linear_batch(queue, arr) == 5
+    queue.finish()
+    for (_, N, _, _, _, ob), want in zip(calls, wants):
+        assert np.array_equal(ob.read(np.uint16, (N,)), want)
+    for b in keep:
+        if b is not None:
+            mil.nnopt_unregister_weight(b)
+
+
+def test_batch_keeps_dependent_calls_in_order(queue):
+    K = 896
+    x = synth_x(60, K)
+    Wa, Wb_ = synth_w(61, K, K), synth_w(62, K, K)
+    qa, sa = mil.quantize_int8(Wa)
+    qb, sb = mil.quantize_int8(Wb_)
+    xb, hb, yb = mil.Buffer.from_host(x), mil.Buffer(K * 2), mil.Buffer(K * 2)
+    A, SA, B, SB = (mil.Buffer.from_host(a) for a in (qa, sa, qb, sb))
+    assert mil.nnopt_register_int8_weight(A, SA, K, K) and mil.nnopt_register_int8_weight(B, SB, K, K)
+    # second call reads the first call's output; third reads x again but writes where the
+    # second reads (write-after-read): order must be kept
+    calls = mil.make_calls([(1, K, K, xb, A, hb), (1, K, K, hb, B, yb), (1, K, K, xb, B, hb)])
+    assert mil.linear_batch(queue, calls) == 3
+    queue.finish()
+    h = O.gemv_i8(x, qa, sa.view(np.uint16))
+    assert np.array_equal(yb.read(np.uint16, (K,)), O.gemv_i8(h.view(np.float16), qb, sb.view(np.uint16)))
+    assert np.array_equal(hb.read(np.uint16, (K,)), O.gemv_i8(x, qb, sb.view(np.uint16)))
+    mil.nnopt_unregister_weight(A)
+    mil.nnopt_unregister_weight(B)
+
+
 @pytest.mark.parametrize("kind", ["i8", "q4"])
 def test_lm_head_full_size(queue, kind):
     """Config 3: W[151936 x 896].  Bit-exact against the oracle on every row."""
