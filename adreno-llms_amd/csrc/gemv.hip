@@ -74,18 +74,39 @@ __device__ __forceinline__ uint16_t f_h(float f) {
     return __half_as_ushort(__float2half_rn(f));
 }
 
-// Two nibbles (bits 0-3 and 16-19 of v) -> two fp16 values (nibble - 8), exact:
-// 0x6400 | n is the half 1024 + n, and (1024 + n) - 1032 is exact.
-__device__ __forceinline__ uint32_t nib_pair(uint32_t v) {
-    uint32_t t = (v & 0x000F000Fu) | 0x64006400u;
-    __half2 h = __builtin_bit_cast(__half2, t);
-    h = __hsub2(h, __builtin_bit_cast(__half2, 0x64086408u));
+// Constants that must sit in registers, not in the instruction stream: gfx950's three-operand
+// encodings take no literal, and a value the compiler can see through gets folded into
+// longer instruction sequences (an fma with a visible -0 addend becomes cvt + cvt + mul).
+struct Consts {
+    uint32_t magic;     // two halves 1024.0
+    float    negzero;   // -0.0f: fma(a, b, -0) == a * b exactly, signed zeros included
+};
+__device__ __forceinline__ Consts make_consts() {
+    Consts c{0x64006400u, -0.0f};
+    asm volatile("" : "+v"(c.magic), "+v"(c.negzero));
+    return c;
+}
+
+// Two nibbles of v -> two fp16 values (nibble - 8), exact.  With the nibbles at bits 0-3 and
+// 16-19, magic | n is the half 1024 + n and (1024 + n) - 1032 is exact; with the nibbles
+// one place up (bits 4-7 and 20-23) magic | (n << 4) is 1024 + 16 n and
+// (1024 + 16 n) / 16 - 72 is exact.  Each pair costs one bit-select and one packed op.
+__device__ __forceinline__ uint32_t nib_pair_lo(uint32_t v, const Consts& c) {
+    const uint32_t t = (v & 0x000F000Fu) | (c.magic & ~0x000F000Fu);
+    const __half2 h = __hsub2(__builtin_bit_cast(__half2, t), __builtin_bit_cast(__half2, 0x64086408u));
+    return __builtin_bit_cast(uint32_t, h);
+}
+__device__ __forceinline__ uint32_t nib_pair_hi(uint32_t v, const Consts& c) {
+    const uint32_t t = (v & 0x00F000F0u) | (c.magic & ~0x00F000F0u);
+    const __half2 h = __hfma2(__builtin_bit_cast(__half2, t), __builtin_bit_cast(__half2, 0x2C002C00u),
+                              __builtin_bit_cast(__half2, 0xD480D480u));      // * 1/16, - 72
     return __builtin_bit_cast(uint32_t, h);
 }
 
 // One virtual lane, one K-iteration.  `scale` is used by Q4 only.
 template <int KIND>
-__device__ __forceinline__ float vlane_step(float acc, const uint32_t* w, const uint32_t* x, float scale) {
+__device__ __forceinline__ float vlane_step(float acc, const uint32_t* w, const uint32_t* x, float scale,
+                                            const Consts& c) {
     if constexpr (KIND == WK_F16) {
         float d = lo_f(x[0]) * lo_f(w[0]);
         d = fmaf(hi_f(x[0]), hi_f(w[0]), d);
@@ -105,9 +126,10 @@ __device__ __forceinline__ float vlane_step(float acc, const uint32_t* w, const 
         return acc + d;
     } else {
         const uint32_t v = w[0];
-        const uint32_t p04 = nib_pair(v), p15 = nib_pair(v >> 4);
-        const uint32_t p26 = nib_pair(v >> 8), p37 = nib_pair(v >> 12);
-        float d = lo_f(x[0]) * lo_f(p04);
+        const uint32_t v8 = v >> 8;
+        const uint32_t p04 = nib_pair_lo(v, c), p15 = nib_pair_hi(v, c);
+        const uint32_t p26 = nib_pair_lo(v8, c), p37 = nib_pair_hi(v8, c);
+        float d = fmaf(lo_f(x[0]), lo_f(p04), c.negzero);
         d = fmaf(hi_f(x[0]), lo_f(p15), d);
         d = fmaf(lo_f(x[1]), lo_f(p26), d);
         d = fmaf(hi_f(x[1]), lo_f(p37), d);
@@ -187,7 +209,9 @@ __device__ __forceinline__ Seg find_segment(const SegList& L, int rb) {
 //
 // PIPE: each wavefront walks several row batches and keeps the next one in flight while it
 // multiplies the current one.  Without PIPE a wavefront is expected to own one batch.
-template <int KIND, int KT, int VL, int EPI, bool PIPE>
+// RB row batches are fetched together, so that narrow rows (Q4, small K) still keep enough
+// bytes in flight per wavefront.
+template <int KIND, int KT, int VL, int EPI, bool PIPE, int RB>
 __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restrict__ x, const SegList L) {
     using T = WT<KIND>;
     constexpr int LPR = kWave / VL, RPW = VL;
@@ -202,6 +226,7 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int g = lane % LPR, r = lane / LPR;
     const int koff = g * VL * T::EPV;
+    const Consts cst = make_consts();
     const int m = blockIdx.y;
     x += static_cast<size_t>(m) * KT;
 
@@ -254,7 +279,7 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
                 const float sf = KIND == WK_Q4 ? h_f(b.s[KIND == WK_Q4 ? j : 0]) : 0.0f;
                 #pragma unroll
                 for (int v = 0; v < VL; ++v)
-                    acc[v] = vlane_step<KIND>(acc[v], &b.w[j][v * T::BPV / 4], &xr[j][v * T::EPV / 2], sf);
+                    acc[v] = vlane_step<KIND>(acc[v], &b.w[j][v * T::BPV / 4], &xr[j][v * T::EPV / 2], sf, cst);
             }
         }
         const float sum = reduce_row<VL>(acc);
@@ -280,17 +305,31 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
             consume(b);
         }
     } else {
-        Batch b0, b1;
-        fetch(b0, rb);
+        // A wavefront owns batches rb, rb + nw, rb + 2 nw, ...; it takes them RB at a time.
+        // A batch index past the end is replaced by the wavefront's first batch (a cached
+        // re-read whose result is dropped), so every fetch issues the same loads.
+        struct Group { Batch b[RB]; };
+        const int first = rb;
+        auto fetch_group = [&](Group& gr, int at) {
+            #pragma unroll
+            for (int u = 0; u < RB; ++u) fetch(gr.b[u], at + u * nw < L.nbatch ? at + u * nw : first);
+        };
+        auto consume_group = [&](const Group& gr, int at) {
+            #pragma unroll
+            for (int u = 0; u < RB; ++u)
+                if (at + u * nw < L.nbatch) consume(gr.b[u]);
+        };
+        const int step = nw * RB;
+        Group g0, g1;
+        fetch_group(g0, rb);
         while (true) {
-            // the prefetch of a batch past the end re-reads the current one (cached, unused)
-            fetch(b1, rb + nw < L.nbatch ? rb + nw : rb);
-            consume(b0);
-            rb += nw;
+            fetch_group(g1, rb + step);
+            consume_group(g0, rb);
+            rb += step;
             if (rb >= L.nbatch) break;
-            fetch(b0, rb + nw < L.nbatch ? rb + nw : rb);
-            consume(b1);
-            rb += nw;
+            fetch_group(g0, rb + step);
+            consume_group(g1, rb);
+            rb += step;
             if (rb >= L.nbatch) break;
         }
     }
@@ -316,6 +355,7 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict_
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int g = lane % LPR, r = lane / LPR;
     const int koff = g * VL * T::EPV;
+    const Consts cst = make_consts();
     const size_t rowb = static_cast<size_t>(K) / T::EPV * T::BPV;
     const int nit = (K + EIT - 1) / EIT;
 
@@ -341,7 +381,7 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict_
                 if constexpr (KIND == WK_Q4) sf = h_f(srow[j * 16]);
                 #pragma unroll
                 for (int v = 0; v < VL; ++v)
-                    acc[v] = vlane_step<KIND>(acc[v], &wr[v * T::BPV / 4], &xr[v * T::EPV / 2], sf);
+                    acc[v] = vlane_step<KIND>(acc[v], &wr[v * T::BPV / 4], &xr[v * T::EPV / 2], sf, cst);
             }
         }
         const float sum = reduce_row<VL>(acc);
@@ -403,6 +443,7 @@ __global__ __launch_bounds__(kBlock) void gate_up_silu_any_k(const uint16_t* __r
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int g = lane % LPR, r = lane / LPR;
     const int koff = g * VL * T::EPV;
+    const Consts cst = make_consts();
     const size_t rowb = static_cast<size_t>(K) / T::EPV * T::BPV;
     const int nit = (K + EIT - 1) / EIT;
     const int nbatch = (N + RPW - 1) / RPW;
@@ -426,8 +467,8 @@ __global__ __launch_bounds__(kBlock) void gate_up_silu_any_k(const uint16_t* __r
                 for (int i = 0; i < XD; ++i) xr[i] = xs[k / 2 + i];
                 #pragma unroll
                 for (int v = 0; v < VL; ++v) {
-                    ag[v] = vlane_step<KIND>(ag[v], &wg[v * T::BPV / 4], &xr[v * T::EPV / 2], 0.0f);
-                    au[v] = vlane_step<KIND>(au[v], &wu[v * T::BPV / 4], &xr[v * T::EPV / 2], 0.0f);
+                    ag[v] = vlane_step<KIND>(ag[v], &wg[v * T::BPV / 4], &xr[v * T::EPV / 2], 0.0f, cst);
+                    au[v] = vlane_step<KIND>(au[v], &wu[v * T::BPV / 4], &xr[v * T::EPV / 2], 0.0f, cst);
                 }
             }
         }
@@ -482,6 +523,12 @@ int pick_vl(WeightKind kind, int M, long rows, int K) {
     return narrowest;
 }
 
+// Row batches a pipelined wavefront fetches at once: enough for about 3.5 KB of weights.
+constexpr int group_size(int kind, int K, int vl) {
+    const int batch_bytes = vl * (K / (kind == WK_Q4 ? 8 : 4)) * (kind == WK_F16 ? 8 : 4);
+    return batch_bytes <= 1280 ? 4 : (batch_bytes <= 2560 ? 2 : 1);
+}
+
 struct Plan {
     SegList L;
     dim3 grid;
@@ -518,10 +565,12 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
     const int K = calls[0].K;
 #define MI_FIXED(KT, PIPE_OK)                                                                            \
     case KT:                                                                                             \
-        if (PIPE_OK && p.pipe)                                                                           \
-            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, PIPE_OK>), p.grid, dim3(kBlock), 0, s, x, p.L); \
-        else                                                                                             \
-            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, false>), p.grid, dim3(kBlock), 0, s, x, p.L);  \
+        if (PIPE_OK && p.pipe) {                                                                         \
+            constexpr int kRB = group_size(KIND, KT, VL);                                                \
+            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, PIPE_OK, kRB>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+        } else {                                                                                         \
+            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, false, 1>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+        }                                                                                                \
         break;
     switch (K) {
         MI_FIXED(576, true)
