@@ -1,14 +1,206 @@
-// Prefill GEMM (M > 1) on MFMA -- placeholder until the tiled kernel lands: reports
-// "unsupported" so that mi_linear runs the batched GEMV for every M.
+// Prefill GEMM for gfx950: out[M,N] = x[M,K] * W[N,K]^T on the matrix cores, with the weight
+// dequantisation fused into the tile load.  fp16 activations, fp16 or per-row int8 weights,
+// fp32 accumulation (v_mfma_f32_32x32x16_f16), fp16 output.
+//
+// Semantics follow the reference's M > 1 path: row i of out is the GEMV of row i of x
+// (LF/src/model.cpp:243-250); for int8 the per-row scale multiplies the fp32 sum once, in the
+// epilogue, as the int8 GEMV does (LF/kernels/gemv_m1_int8.cl:69-77).  int8 weights convert
+// exactly to fp16, so every product is exact in fp32; only the order of the fp32 additions
+// differs from the GEMV kernels (results agree to fp32 rounding, not bit for bit).
+//
+// Both operands are K-contiguous, so a block stages a BM x 64 tile of x and a BN x 64 tile of W
+// through LDS (rows padded to 72 halves: 16-byte reads of 8 consecutive rows then fall in
+// 8 different bank groups) while the loads of the next K-tile are already in flight in
+// registers.  Four wavefronts per block, each owning a WM x WN sub-tile as (WM/32) x (WN/32)
+// accumulators of 32 x 32.
 #include "common.h"
+#include <hip/hip_fp16.h>
 
 namespace mi {
+namespace {
 
-bool gemm_supported(WeightKind, int, int, int) { return false; }
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-bool launch_gemm(hipStream_t, WeightKind, int, int, int, const void*, const void*, const void*, void*) {
-    MI_ERROR_FMT("gemm: not built");
-    return false;
+constexpr int kKT = 64;            // K-tile, elements
+constexpr int kLd = kKT + 8;       // LDS row stride, halves
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ uint16_t to_half_bits(float f) {
+    asm volatile("" : "+v"(f));    // round the fp32 value first, then convert (two roundings, as the GEMV path)
+    return __half_as_ushort(__float2half_rn(f));
+}
+
+// Four int8 in one dword -> four fp16 (two dwords), exact: byte ^ 0x80 is q + 128, the byte
+// permute builds the halves 1024 + (q + 128), and subtracting 1152 leaves q.
+__device__ __forceinline__ void i8x4_to_h4(uint32_t v, uint32_t& lo, uint32_t& hi) {
+    const uint32_t u = v ^ 0x80808080u;
+    const uint32_t a = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
+    const uint32_t b = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
+    const __half2 k = __builtin_bit_cast(__half2, 0x64806480u);               // 1152, 1152
+    lo = __builtin_bit_cast(uint32_t, __hsub2(__builtin_bit_cast(__half2, a), k));
+    hi = __builtin_bit_cast(uint32_t, __hsub2(__builtin_bit_cast(__half2, b), k));
+}
+
+template <int BM, int BN, int WM, int WN, int KIND>
+__global__ __launch_bounds__(kThreads) void gemm_kernel(const uint16_t* __restrict__ X,
+                                                        const uint8_t* __restrict__ W,
+                                                        const uint16_t* __restrict__ scale,
+                                                        uint16_t* __restrict__ out, int M, int N, int K) {
+    static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per block");
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int A_CHUNKS = BM * (kKT / 8) / kThreads;                      // 16-byte chunks of x per thread
+    constexpr int B_BYTES = KIND == WK_I8 ? 1 : 2;
+    constexpr int B_CPR = kKT * B_BYTES / 16;                                // 16-byte chunks per W row and K-tile
+    constexpr int B_CHUNKS = BN * B_CPR / kThreads;
+    static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1, "tile too small for 256 threads");
+
+    __shared__ __attribute__((aligned(16))) uint16_t As[BM * kLd];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * kLd];
+
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int wm = wave / (BN / WN), wn = wave % (BN / WN);
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int gk = lane / 32, li = lane % 32;
+
+    floatx16 acc[TM][TN];
+    #pragma unroll
+    for (int t = 0; t < TM; ++t)
+        #pragma unroll
+        for (int u = 0; u < TN; ++u)
+            #pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][u][r] = 0.0f;
+
+    u32x4 ra[A_CHUNKS], rb[B_CHUNKS];
+    auto load_tile = [&](int k0) {
+        #pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) {
+            const int c = tid + i * kThreads, row = c / (kKT / 8), kc = c % (kKT / 8);
+            const int m = m0 + row;
+            if (m < M) ra[i] = *reinterpret_cast<const u32x4*>(X + static_cast<size_t>(m) * K + k0 + kc * 8);
+            else ra[i] = u32x4{0u, 0u, 0u, 0u};
+        }
+        #pragma unroll
+        for (int i = 0; i < B_CHUNKS; ++i) {
+            const int c = tid + i * kThreads, row = c / B_CPR, kc = c % B_CPR;
+            const int n = n0 + row;
+            if (n < N)
+                rb[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+                    W + (static_cast<size_t>(n) * K + k0) * B_BYTES + kc * 16));
+            else rb[i] = u32x4{0u, 0u, 0u, 0u};
+        }
+    };
+    auto store_tile = [&]() {
+        #pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) {
+            const int c = tid + i * kThreads, row = c / (kKT / 8), kc = c % (kKT / 8);
+            *reinterpret_cast<u32x4*>(&As[row * kLd + kc * 8]) = ra[i];
+        }
+        #pragma unroll
+        for (int i = 0; i < B_CHUNKS; ++i) {
+            const int c = tid + i * kThreads, row = c / B_CPR, kc = c % B_CPR;
+            if constexpr (KIND == WK_I8) {
+                uint32_t h[8];
+                i8x4_to_h4(rb[i].x, h[0], h[1]);
+                i8x4_to_h4(rb[i].y, h[2], h[3]);
+                i8x4_to_h4(rb[i].z, h[4], h[5]);
+                i8x4_to_h4(rb[i].w, h[6], h[7]);
+                *reinterpret_cast<u32x4*>(&Bs[row * kLd + kc * 16]) = u32x4{h[0], h[1], h[2], h[3]};
+                *reinterpret_cast<u32x4*>(&Bs[row * kLd + kc * 16 + 8]) = u32x4{h[4], h[5], h[6], h[7]};
+            } else {
+                *reinterpret_cast<u32x4*>(&Bs[row * kLd + kc * 8]) = rb[i];
+            }
+        }
+    };
+
+    load_tile(0);
+    for (int k0 = 0; k0 < K; k0 += kKT) {
+        __syncthreads();                       // everyone is done reading the previous tile
+        store_tile();
+        __syncthreads();
+        if (k0 + kKT < K) load_tile(k0 + kKT); // in flight while the matrix cores work
+        #pragma unroll
+        for (int kk = 0; kk < kKT / 16; ++kk) {
+            // lane group gk supplies k = 32 gk + 8 kk .. +7 of the tile, for both operands
+            const int kcol = 32 * gk + 8 * kk;
+            half8 a[TM], b[TN];
+            #pragma unroll
+            for (int t = 0; t < TM; ++t)
+                a[t] = *reinterpret_cast<const half8*>(&As[(wm * WM + t * 32 + li) * kLd + kcol]);
+            #pragma unroll
+            for (int u = 0; u < TN; ++u)
+                b[u] = *reinterpret_cast<const half8*>(&Bs[(wn * WN + u * 32 + li) * kLd + kcol]);
+            #pragma unroll
+            for (int t = 0; t < TM; ++t)
+                #pragma unroll
+                for (int u = 0; u < TN; ++u)
+                    acc[t][u] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[t], b[u], acc[t][u], 0, 0, 0);
+        }
+    }
+
+    // D[i][j]: j = lane % 32 (a W row, i.e. an output column), i = 8 (r / 4) + 4 (lane / 32) + r % 4.
+    #pragma unroll
+    for (int u = 0; u < TN; ++u) {
+        const int n = n0 + wn * WN + u * 32 + li;
+        if (n >= N) continue;
+        float s = 1.0f;
+        if constexpr (KIND == WK_I8) s = __half2float(__ushort_as_half(scale[n]));
+        #pragma unroll
+        for (int t = 0; t < TM; ++t) {
+            #pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * WM + t * 32 + 8 * (r / 4) + 4 * gk + r % 4;
+                if (m < M) {
+                    const float v = KIND == WK_I8 ? acc[t][u][r] * s : acc[t][u][r];
+                    out[static_cast<size_t>(m) * N + n] = to_half_bits(v);
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WM, int WN>
+bool launch_tile(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x, const void* W,
+                 const void* scale, void* out) {
+    const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, 1);
+    const auto* xp = static_cast<const uint16_t*>(x);
+    const auto* wp = static_cast<const uint8_t*>(W);
+    const auto* sp = static_cast<const uint16_t*>(scale);
+    auto* op = static_cast<uint16_t*>(out);
+    if (kind == WK_I8)
+        hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, WK_I8>), grid, dim3(kThreads), 0, s, xp, wp, sp, op, M, N, K);
+    else
+        hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, WK_F16>), grid, dim3(kThreads), 0, s, xp, wp, sp, op, M, N, K);
+    return MI_HIP_OK(hipGetLastError());
+}
+
+inline long tiles(int M, int N, int bm, int bn) {
+    return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+}
+
+}  // namespace
+
+bool gemm_supported(WeightKind kind, int M, int N, int K) {
+    return (kind == WK_I8 || kind == WK_F16) && M >= 16 && N >= 1 && K >= kKT && K % kKT == 0;
+}
+
+bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x, const void* W,
+                 const void* scale, void* out) {
+    if (!gemm_supported(kind, M, N, K)) {
+        MI_ERROR_FMT("gemm: unsupported kind=%d M=%d N=%d K=%d", static_cast<int>(kind), M, N, K);
+        return false;
+    }
+    if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(W) % 16 ||
+        (kind == WK_I8 && !scale)) {
+        MI_ERROR_FMT("gemm: x and W must be 16-byte aligned, int8 needs a scale");
+        return false;
+    }
+    // Largest tile that still yields about one block per CU.
+    const long want = device_info().cus;
+    if (M > 64 && tiles(M, N, 256, 128) >= want) return launch_tile<256, 128, 128, 64>(s, kind, M, N, K, x, W, scale, out);
+    if (M > 64 && tiles(M, N, 128, 128) >= want) return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);
+    return launch_tile<64, 64, 32, 32>(s, kind, M, N, K, x, W, scale, out);
 }
 
 }  // namespace mi

@@ -1,0 +1,128 @@
+"""GPU parity of the prefill GEMM (M > 1 on the matrix cores), through the C ABI.
+
+Reference semantics: row i of out is the GEMV of row i of x (the reference's quantised
+prefill is a loop of M = 1 calls, LF/src/model.cpp:243-250).  The MFMA kernel sums in a
+different fp32 order than the GEMV kernels, so the bar here is the stated tolerance
+(max-abs/rel 1e-3, cosine >= 0.9999), tightened to "at most 1 fp16 ulp apart"; the batched
+GEMV mode of the same entry point stays bit-exact."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from helpers import assert_tolerance, mil, synth_w, synth_x
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def queue():
+    assert mil.lib().mi_init(0) == 1, "no gfx950 device"
+    q = mil.Queue()
+    yield q
+    q.finish()
+
+
+def _ulp_apart(a_u16, b_u16):
+    """|a - b| in units of the fp16 spacing at max(|b|, 1e-3 max|b|): outputs that cancel to
+    almost zero carry the absolute fp32 rounding error of sums of much larger terms, so their
+    own (tiny) fp16 spacing is not the yardstick."""
+    a = a_u16.view(np.float16).astype(np.float64)
+    b = b_u16.view(np.float16).astype(np.float64)
+    mag = np.maximum(np.abs(b), 1e-3 * np.abs(b).max())
+    step = np.spacing(mag.astype(np.float16)).astype(np.float64)
+    return np.abs(a - b) / step
+
+
+def _gemm(queue, M, N, K, X, W_host, scale_host, kind):
+    xb, wb = mil.Buffer.from_host(X), mil.Buffer.from_host(W_host)
+    sb = mil.Buffer.from_host(scale_host) if scale_host is not None else None
+    if kind == "i8":
+        assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+    pad = 128
+    guard = np.full(M * N + 2 * pad, 0x7BCD, np.uint16)
+    ob = mil.Buffer.from_host(guard)
+    assert mil.pytorch_linear(queue, M, N, K, xb, wb, ob.ptr + 2 * pad)
+    queue.finish()
+    full = ob.read(np.uint16, guard.shape)
+    assert np.all(full[:pad] == 0x7BCD) and np.all(full[-pad:] == 0x7BCD), "wrote outside out[M,N]"
+    mil.nnopt_unregister_weight(wb)
+    return full[pad:-pad].reshape(M, N)
+
+
+@pytest.mark.parametrize("M", [16, 64, 100, 512])
+@pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (200, 128), (130, 576)])
+def test_int8_gemm_matches_rows_of_gemv(queue, M, N, K):
+    print(f"int8 gemm M={M} N={N} K={K}", flush=True)
+    W, X = synth_w(700 + N, N, K), synth_x(800 + M, M, K)
+    q, s = mil.quantize_int8(W)
+    got = _gemm(queue, M, N, K, X, q, s, "i8")
+    want = O.gemm_i8(X, q, s.view(np.uint16))
+    assert_tolerance(got.view(np.float16), want.view(np.float16))
+    d = _ulp_apart(got, want)
+    assert d.max() <= 1, f"max {d.max()} fp16 steps apart"
+    assert np.mean(got == want) > 0.99
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 4864, 896), (256, 896, 4864), (33, 200, 128)])
+def test_fp16_gemm_matches_rows_of_gemv(queue, M, N, K):
+    W, X = synth_w(900 + N, N, K), synth_x(901 + M, M, K)
+    got = _gemm(queue, M, N, K, X, W, None, "f16")
+    want = O.gemm_f16(X, W)
+    assert_tolerance(got.view(np.float16), want.view(np.float16))
+    assert _ulp_apart(got, want).max() <= 1
+
+
+def test_gemm_exact_on_integer_data(queue):
+    # small integers: every partial sum is exact in fp32, so any summation order gives the same bits
+    rng = np.random.default_rng(3)
+    M, N, K = 96, 192, 256
+    q = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    X = rng.integers(-3, 4, (M, K)).astype(np.float16)
+    s = (2.0 ** rng.integers(-10, -6, N)).astype(np.float16)
+    got = _gemm(queue, M, N, K, X, q, s, "i8")
+    want = ((X.astype(np.int64) @ q.astype(np.int64).T).astype(np.float64) * s.astype(np.float64)).astype(np.float16)
+    assert np.array_equal(got.view(np.float16), want)
+    assert np.array_equal(got, O.gemm_i8(X, q, s.view(np.uint16)))
+
+
+def test_gemm_unit_rows_pick_weight_columns(queue):
+    # x rows are unit vectors: out[i, :] must be the dequantised column k_i of W (index check)
+    M, N, K = 64, 320, 896
+    W = synth_w(910, N, K)
+    q, s = mil.quantize_int8(W)
+    ks = (np.arange(M) * 37 + 5) % K
+    X = np.zeros((M, K), np.float16)
+    X[np.arange(M), ks] = 1.0
+    got = _gemm(queue, M, N, K, X, q, s, "i8").view(np.float16)
+    want = (q[:, ks].T.astype(np.float32) * s.astype(np.float32)[None, :]).astype(np.float16)
+    assert np.array_equal(got, want)
+
+
+def test_prefill_size_rows_sampled(queue):
+    """Config 5 at M = 2048: every sampled row of out equals the GEMV of that row of x."""
+    M, N, K = 2048, 4864, 896
+    W, X = synth_w(920, N, K), synth_x(921, M, K)
+    q, s = mil.quantize_int8(W)
+    got = _gemm(queue, M, N, K, X, q, s, "i8")
+    rows = np.array([0, 1, 31, 32, 127, 128, 255, 256, 1000, 1023, 1024, 2046, 2047])
+    for r in rows:
+        want = O.gemv_i8(X[r], q, s.view(np.uint16))
+        assert _ulp_apart(got[r], want).max() <= 1, f"row {r}"
+    # linearity in x: scaling a row of x by 2 scales the output row by 2 exactly
+    X2 = X.copy()
+    X2[5] = X[5] * np.float16(2.0)
+    got2 = _gemm(queue, M, N, K, X2, q, s, "i8")
+    assert np.array_equal(got2[5].view(np.float16), got[5].view(np.float16) * np.float16(2.0))
+    assert np.array_equal(got2[6], got[6])
+
+
+def test_batched_gemv_mode_stays_bit_exact(queue):
+    M, N, K = 32, 896, 896
+    W, X = synth_w(930, N, K), synth_x(931, M, K)
+    q, s = mil.quantize_int8(W)
+    mil.lib().mi_set_gemm_mode(1)
+    try:
+        got = _gemm(queue, M, N, K, X, q, s, "i8")
+    finally:
+        mil.lib().mi_set_gemm_mode(0)
+    assert np.array_equal(got, O.gemm_i8(X, q, s.view(np.uint16)))
