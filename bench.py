@@ -204,6 +204,29 @@ def main():
         detail["c3_int8_gemv_151936x896"] = {"us": roofline["us_per_launch"], "GBps": roofline["achieved"],
                                              "frac_hbm": roofline["frac"], "bytes": lm_bytes}
 
+    # ---- config 5: prefill GEMM with fused int8 dequant on the matrix cores ---------------
+    if not args.no_detail:
+        MFMA_PEAK_TFLOPS = 2500.0
+        for (N, K) in ((INTER, H), (H, INTER)):
+            w = mil.synth_normal_f16(77, 0.02, (N, K))
+            qh, sh = mil.quantize_int8(w)
+            wb, sb = mil.Buffer.from_host(qh), mil.Buffer.from_host(sh)
+            assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+            for M in (16, 64, 512, 2048):
+                xb = mil.Buffer.from_host(mil.synth_normal_f16(78, 1.0, (M, K)))
+                ob = mil.Buffer(M * N * 2)
+                arr = mil.make_calls([(M, N, K, xb, wb, ob)] * 20)
+                mil.linear_batch(queue, arr)
+                ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 5) / 20
+                flop = 2.0 * M * N * K
+                nbytes = 2 * M * K + N * K + 2 * N + 2 * M * N
+                detail[f"c5_int8_gemm_M{M}_N{N}_K{K}"] = {
+                    "us": round(ms * 1e3, 2), "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 1),
+                    "frac_mfma_fp16_peak": round(flop / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                    "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                    "frac_hbm": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+            mil.nnopt_unregister_weight(wb)
+
     # ---- CPU baseline: the oracle on a bounded sample of the same sweep -------------------
     cpu = None
     if not args.no_cpu:
