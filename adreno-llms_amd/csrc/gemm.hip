@@ -10,8 +10,8 @@
 //
 // Both operands are K-contiguous, so a block stages a BM x 64 tile of x and a BN x 64 tile of W
 // through LDS (rows padded to 72 halves: 16-byte reads of 8 consecutive rows then fall in
-// 8 different bank groups) while the loads of the next K-tile are already in flight in
-// registers.  Four wavefronts per block, each owning a WM x WN sub-tile as (WM/32) x (WN/32)
+// 8 different bank groups; two LDS stages) while the loads of the next three K-tiles are
+// already in flight in registers.  Four wavefronts per block, each owning a WM x WN sub-tile as (WM/32) x (WN/32)
 // accumulators of 32 x 32.
 #include "common.h"
 #include <hip/hip_fp16.h>
@@ -56,8 +56,11 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const uint16_t* __restri
     constexpr int B_CHUNKS = BN * B_CPR / kThreads;
     static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1, "tile too small for 256 threads");
 
-    __shared__ __attribute__((aligned(16))) uint16_t As[BM * kLd];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * kLd];
+    // Two LDS stages (x tile then W tile in each) and kStages register stages: the global
+    // loads of K-tile i + kStages are issued while tile i is multiplied, which is what hides
+    // the HBM / L2 latency (one tile ahead is far too short for it).
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    constexpr int kStageHalves = (BM + BN) * kLd;
 
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int wm = wave / (BN / WN), wn = wave % (BN / WN);
@@ -72,54 +75,45 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const uint16_t* __restri
             #pragma unroll
             for (int r = 0; r < 16; ++r) acc[t][u][r] = 0.0f;
 
-    u32x4 ra[A_CHUNKS], rb[B_CHUNKS];
-    auto load_tile = [&](int k0) {
+    struct Regs { u32x4 a[A_CHUNKS]; u32x4 b[B_CHUNKS]; };
+    auto load_tile = [&](Regs& R, int k0) {
         #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
             const int c = tid + i * kThreads, row = c / (kKT / 8), kc = c % (kKT / 8);
-            const int m = m0 + row;
-            if (m < M) ra[i] = *reinterpret_cast<const u32x4*>(X + static_cast<size_t>(m) * K + k0 + kc * 8);
-            else ra[i] = u32x4{0u, 0u, 0u, 0u};
+            const int m = m0 + row < M ? m0 + row : M - 1;          // rows past M are never stored
+            R.a[i] = *reinterpret_cast<const u32x4*>(X + static_cast<size_t>(m) * K + k0 + kc * 8);
         }
         #pragma unroll
         for (int i = 0; i < B_CHUNKS; ++i) {
             const int c = tid + i * kThreads, row = c / B_CPR, kc = c % B_CPR;
-            const int n = n0 + row;
-            if (n < N)
-                rb[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
-                    W + (static_cast<size_t>(n) * K + k0) * B_BYTES + kc * 16));
-            else rb[i] = u32x4{0u, 0u, 0u, 0u};
+            const int n = n0 + row < N ? n0 + row : N - 1;
+            R.b[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+                W + (static_cast<size_t>(n) * K + k0) * B_BYTES + kc * 16));
         }
     };
-    auto store_tile = [&]() {
+    auto store_tile = [&](const Regs& R, uint16_t* As, uint16_t* Bs) {
         #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
             const int c = tid + i * kThreads, row = c / (kKT / 8), kc = c % (kKT / 8);
-            *reinterpret_cast<u32x4*>(&As[row * kLd + kc * 8]) = ra[i];
+            *reinterpret_cast<u32x4*>(&As[row * kLd + kc * 8]) = R.a[i];
         }
         #pragma unroll
         for (int i = 0; i < B_CHUNKS; ++i) {
             const int c = tid + i * kThreads, row = c / B_CPR, kc = c % B_CPR;
             if constexpr (KIND == WK_I8) {
                 uint32_t h[8];
-                i8x4_to_h4(rb[i].x, h[0], h[1]);
-                i8x4_to_h4(rb[i].y, h[2], h[3]);
-                i8x4_to_h4(rb[i].z, h[4], h[5]);
-                i8x4_to_h4(rb[i].w, h[6], h[7]);
+                i8x4_to_h4(R.b[i].x, h[0], h[1]);
+                i8x4_to_h4(R.b[i].y, h[2], h[3]);
+                i8x4_to_h4(R.b[i].z, h[4], h[5]);
+                i8x4_to_h4(R.b[i].w, h[6], h[7]);
                 *reinterpret_cast<u32x4*>(&Bs[row * kLd + kc * 16]) = u32x4{h[0], h[1], h[2], h[3]};
                 *reinterpret_cast<u32x4*>(&Bs[row * kLd + kc * 16 + 8]) = u32x4{h[4], h[5], h[6], h[7]};
             } else {
-                *reinterpret_cast<u32x4*>(&Bs[row * kLd + kc * 8]) = rb[i];
+                *reinterpret_cast<u32x4*>(&Bs[row * kLd + kc * 8]) = R.b[i];
             }
         }
     };
-
-    load_tile(0);
-    for (int k0 = 0; k0 < K; k0 += kKT) {
-        __syncthreads();                       // everyone is done reading the previous tile
-        store_tile();
-        __syncthreads();
-        if (k0 + kKT < K) load_tile(k0 + kKT); // in flight while the matrix cores work
+    auto multiply = [&](const uint16_t* As, const uint16_t* Bs) {
         #pragma unroll
         for (int kk = 0; kk < kKT / 16; ++kk) {
             // lane group gk supplies k = 32 gk + 8 kk .. +7 of the tile, for both operands
@@ -137,7 +131,32 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const uint16_t* __restri
                 for (int u = 0; u < TN; ++u)
                     acc[t][u] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[t], b[u], acc[t][u], 0, 0, 0);
         }
+    };
+
+    const int nk = K / kKT;
+    Regs R0, R1, R2;
+    load_tile(R0, 0);
+    load_tile(R1, (1 < nk ? 1 : nk - 1) * kKT);
+    load_tile(R2, (2 < nk ? 2 : nk - 1) * kKT);
+    // One step: tile i goes registers -> LDS stage i % 2; one barrier publishes it (and, being
+    // the second barrier since stage i % 2 was last read, also guards the overwrite); the
+    // freed registers take tile i + 3; the matrix cores run on tile i.
+#define MI_GEMM_STEP(R)                                                        \
+    {                                                                          \
+        uint16_t* As = lds + (i & 1) * kStageHalves;                           \
+        uint16_t* Bs = As + BM * kLd;                                          \
+        store_tile(R, As, Bs);                                                 \
+        __syncthreads();                                                       \
+        load_tile(R, (i + 3 < nk ? i + 3 : nk - 1) * kKT);                     \
+        multiply(As, Bs);                                                      \
+        if (++i >= nk) break;                                                  \
     }
+    for (int i = 0;;) {
+        MI_GEMM_STEP(R0)
+        MI_GEMM_STEP(R1)
+        MI_GEMM_STEP(R2)
+    }
+#undef MI_GEMM_STEP
 
     // D[i][j]: j = lane % 32 (a W row, i.e. an output column), i = 8 (r / 4) + 4 (lane / 32) + r % 4.
     #pragma unroll
@@ -168,10 +187,26 @@ bool launch_tile(hipStream_t s, WeightKind kind, int M, int N, int K, const void
     const auto* wp = static_cast<const uint8_t*>(W);
     const auto* sp = static_cast<const uint16_t*>(scale);
     auto* op = static_cast<uint16_t*>(out);
-    if (kind == WK_I8)
-        hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, WK_I8>), grid, dim3(kThreads), 0, s, xp, wp, sp, op, M, N, K);
-    else
-        hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, WK_F16>), grid, dim3(kThreads), 0, s, xp, wp, sp, op, M, N, K);
+    constexpr size_t lds_bytes = 2u * (BM + BN) * kLd * sizeof(uint16_t);
+    // more than 64 KB of LDS per block has to be asked for once per kernel
+    static bool raised_i8 = false, raised_f16 = false;
+    if (kind == WK_I8) {
+        auto* kern = gemm_kernel<BM, BN, WM, WN, WK_I8>;
+        if (lds_bytes > 65536 && !raised_i8) {
+            if (!MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes))) return false;
+            raised_i8 = true;
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, s, xp, wp, sp, op, M, N, K);
+    } else {
+        auto* kern = gemm_kernel<BM, BN, WM, WN, WK_F16>;
+        if (lds_bytes > 65536 && !raised_f16) {
+            if (!MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes))) return false;
+            raised_f16 = true;
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, s, xp, wp, sp, op, M, N, K);
+    }
     return MI_HIP_OK(hipGetLastError());
 }
 
@@ -196,10 +231,10 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
         MI_ERROR_FMT("gemm: x and W must be 16-byte aligned, int8 needs a scale");
         return false;
     }
-    // Largest tile that still yields about one block per CU.
-    const long want = device_info().cus;
-    if (M > 64 && tiles(M, N, 256, 128) >= want) return launch_tile<256, 128, 128, 64>(s, kind, M, N, K, x, W, scale, out);
-    if (M > 64 && tiles(M, N, 128, 128) >= want) return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);
+    // 128 x 128 tiles once they fill every CU twice over (two blocks are resident per CU);
+    // below that the 64 x 64 tile spreads the work over more CUs and wins (measured).
+    if (M > 64 && tiles(M, N, 128, 128) >= 2L * device_info().cus)
+        return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);
     return launch_tile<64, 64, 32, 32>(s, kind, M, N, K, x, W, scale, out);
 }
 

@@ -32,6 +32,10 @@ H, INTER, KV, VOCAB, LAYERS = 896, 4864, 128, 151936, 24
 LAYER_SHAPES = [("q", H, H), ("k", KV, H), ("v", KV, H), ("o", H, H),
                 ("gate", INTER, H), ("up", INTER, H), ("down", H, INTER)]
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the lm_head int8 GEMV kernel, from rocprofv3 FETCH_SIZE and WRITE_SIZE
+# (separate counter runs of this script, scaled by what the same counters read for a
+# device-to-device copy of known size; profiles/gemv_int8_lm_head_hbm_traffic.txt).
+LM_HEAD_I8_TRAFFIC_BYTES = 142133000
 
 
 def algo_bytes_i8(N, K):
@@ -154,7 +158,7 @@ def main():
     achieved = lm_bytes / (ms_lm * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "gemv int8 K=896 (lm_head, N=151936)", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": None, "us_per_launch": round(ms_lm * 1e3, 2), "bytes_per_launch": lm_bytes}
+                "traffic": LM_HEAD_I8_TRAFFIC_BYTES, "us_per_launch": round(ms_lm * 1e3, 2), "bytes_per_launch": lm_bytes}
 
     # ---- per-config detail -------------------------------------------------------------------
     detail = {"decode_step_us_stream": round(ms_stream * 1e3, 1), "decode_step_us_graph": None if args.no_graph else round(ms_graph * 1e3, 1),
