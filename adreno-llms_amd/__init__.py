@@ -55,6 +55,7 @@ _SIGNATURES = {
     "mi_dequant_int8_to_fp16": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "mi_unpack_q4_to_int8": (_i, [_vp, _vp, _i, _i, _vp]),
     "mi_set_gemm_mode": (None, [_i]),
+    "mi_set_gemv_mode": (None, [_i]),
     "mi_quantize_int8": (_i, [_vp, _i, _i, _vp, _vp]),
     "mi_quantize_q4": (_i, [_vp, _i, _i, _vp, _vp]),
     "mi_f16_to_f32": (C.c_float, [C.c_uint16]),

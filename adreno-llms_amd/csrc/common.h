@@ -30,6 +30,9 @@ struct DeviceInfo {
     char arch[64] = {0};
 };
 const DeviceInfo& device_info();
+// 0 = every GEMV evaluates the reference kernels' sum in their order (bit-exact);
+// 1 = Q4 may use the throughput kernel (same fp32 sum, other order).
+int gemv_mode();
 
 // M rows of x (stride K) against one W; y rows have stride N.
 struct GemvCall {

@@ -335,6 +335,151 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     }
 }
 
+// ---- Q4, throughput variant --------------------------------------------------------
+//
+// The exact Q4 kernel above is bound by the vector ALU, not by HBM: reproducing the
+// reference's sum needs one fp32 fma per weight after the nibble has become a number.
+// This variant keeps the result inside the stated tolerance (max-abs/rel 1e-3, cosine
+// 0.9999; the sum is still fp32, only its order changes) at about half the instructions:
+//   - a nibble pair masked in place is read as two fp16 SUBNORMALS, n * 2^-24 (pairs at
+//     bits 0-3/16-19) or n * 2^-20 (pairs at bits 4-7/20-23): no conversion at all;
+//   - v_dot2_f32_f16 multiplies a pair by the matching pair of activations and accumulates
+//     in fp32, two weights per instruction (the activations are held pre-paired);
+//   - the "- 8" of every weight is applied once per 32-weight block as -8 * sum(x), and the
+//     block scale multiplies the block sum once.
+// 16 lanes still share a row and a wavefront still streams row batches of 4 rows with the
+// same double-buffered fetch; each lane owns one scale block per K-iteration.
+template <int KT, int EPI, bool PIPE, int RB>
+__global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restrict__ x, const SegList L) {
+    constexpr int EIT = 512;                            // elements per K-iteration (16 lanes x 32)
+    constexpr int NIT = (KT + EIT - 1) / EIT;
+    constexpr int ROWB = KT / 2;
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int g = lane % 16, r = lane / 16;
+    const int koff = g * 32;
+    const int m = blockIdx.y;
+    x += static_cast<size_t>(m) * KT;
+
+    // xp[j][4 d + i]: activations paired for dword d of the lane's 16 weight bytes:
+    // i = 0: (x0, x4), 1: (x1, x5), 2: (x2, x6), 3: (x3, x7) of elements 8 d .. 8 d + 7.
+    uint32_t xp[NIT][16];
+    float m8sx[NIT];                                    // -8 * sum of the block's activations
+    #pragma unroll
+    for (int j = 0; j < NIT; ++j) {
+        uint32_t raw[16];
+        if (j * EIT + koff < KT) load_dwords<16, false>(raw, x + j * EIT + koff);
+        else {
+            #pragma unroll
+            for (int i = 0; i < 16; ++i) raw[i] = 0u;
+        }
+        float sx = 0.0f;
+        #pragma unroll
+        for (int i = 0; i < 16; ++i) sx += lo_f(raw[i]) + hi_f(raw[i]);
+        m8sx[j] = -8.0f * sx;
+        #pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            xp[j][4 * d + 0] = __builtin_amdgcn_perm(raw[4 * d + 2], raw[4 * d + 0], 0x05040100u);
+            xp[j][4 * d + 1] = __builtin_amdgcn_perm(raw[4 * d + 2], raw[4 * d + 0], 0x07060302u);
+            xp[j][4 * d + 2] = __builtin_amdgcn_perm(raw[4 * d + 3], raw[4 * d + 1], 0x05040100u);
+            xp[j][4 * d + 3] = __builtin_amdgcn_perm(raw[4 * d + 3], raw[4 * d + 1], 0x07060302u);
+        }
+    }
+
+    struct Batch {
+        uint32_t w[NIT][4];
+        uint16_t s[NIT];
+        uint16_t res;
+        uint16_t* yrow;
+    };
+    auto fetch = [&](Batch& b, int rb) {
+        const Seg sg = find_segment(L, rb);
+        const int row = (rb - sg.first) * 4 + r;
+        const bool valid = row < sg.N;
+        const int rowc = valid ? row : sg.N - 1;
+        uint16_t* yp = sg.y + static_cast<size_t>(m) * sg.N + rowc;
+        b.yrow = valid ? yp : nullptr;
+        if constexpr (EPI == EPI_ADD) b.res = *yp;
+        const uint8_t* wrow = sg.W + static_cast<size_t>(rowc) * ROWB;
+        #pragma unroll
+        for (int j = 0; j < NIT; ++j) {
+            const bool active = j * EIT + koff < KT;
+            load_dwords<4, true>(b.w[j], wrow + (active ? j * 256 + g * 16 : 0));
+            b.s[j] = sg.sc[static_cast<size_t>(rowc) * (KT / 32) + (active ? j * 16 + g : 0)];
+        }
+    };
+    auto consume = [&](const Batch& b) {
+        float acc = 0.0f;
+        #pragma unroll
+        for (int j = 0; j < NIT; ++j) {
+            if (j * EIT + koff < KT) {
+                float da = 0.0f, db = 0.0f;
+                #pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const uint32_t v = b.w[j][d], v8 = v >> 8;
+                    da = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xp[j][4 * d + 0]),
+                                                __builtin_bit_cast(h2, v & 0x000F000Fu), da, false);
+                    db = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xp[j][4 * d + 1]),
+                                                __builtin_bit_cast(h2, v & 0x00F000F0u), db, false);
+                    da = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xp[j][4 * d + 2]),
+                                                __builtin_bit_cast(h2, v8 & 0x000F000Fu), da, false);
+                    db = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xp[j][4 * d + 3]),
+                                                __builtin_bit_cast(h2, v8 & 0x00F000F0u), db, false);
+                }
+                // sum over the block of x * (n - 8) = 2^24 da + 2^20 db - 8 sum(x)
+                const float blk = fmaf(da, 16777216.0f, fmaf(db, 1048576.0f, m8sx[j]));
+                acc = fmaf(blk, h_f(b.s[j]), acc);
+            }
+        }
+        acc = add_from_above<8>(acc);
+        acc = add_from_above<4>(acc);
+        acc = add_from_above<2>(acc);
+        acc = add_from_above<1>(acc);
+        if (g == 0 && b.yrow) {
+            const float out = EPI == EPI_ADD ? acc + h_f(b.res) : acc;
+            *b.yrow = f_h(out);
+        }
+    };
+
+    const int nw = gridDim.x * kWavesPerBlock;
+    int rb = blockIdx.x * kWavesPerBlock + wave;
+    if (rb >= L.nbatch) return;
+    if constexpr (!PIPE) {
+        for (; rb < L.nbatch; rb += nw) {
+            Batch b;
+            fetch(b, rb);
+            consume(b);
+        }
+    } else {
+        struct Group { Batch b[RB]; };
+        const int first = rb;
+        auto fetch_group = [&](Group& gr, int at) {
+            #pragma unroll
+            for (int u = 0; u < RB; ++u) fetch(gr.b[u], at + u * nw < L.nbatch ? at + u * nw : first);
+        };
+        auto consume_group = [&](const Group& gr, int at) {
+            #pragma unroll
+            for (int u = 0; u < RB; ++u)
+                if (at + u * nw < L.nbatch) consume(gr.b[u]);
+        };
+        const int step = nw * RB;
+        Group g0, g1;
+        fetch_group(g0, rb);
+        while (true) {
+            fetch_group(g1, rb + step);
+            consume_group(g0, rb);
+            rb += step;
+            if (rb >= L.nbatch) break;
+            fetch_group(g0, rb + step);
+            consume_group(g1, rb);
+            rb += step;
+            if (rb >= L.nbatch) break;
+        }
+    }
+}
+
 // ---- K known at run time: x is staged once per block in LDS ------------------------
 template <int KIND, int VL, int EPI>
 __global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict__ x, const SegList L, int K) {
@@ -587,6 +732,34 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
     return MI_HIP_OK(hipGetLastError());
 }
 
+// Throughput variant of Q4 (see gemv_q4_fast): K known at compile time and a whole number of
+// 32-weight blocks per lane, i.e. the 16-byte lane tile.
+template <int EPI>
+bool launch_q4_fast(hipStream_t s, const GemvCall* calls, int n, bool* taken) {
+    const int K = calls[0].K;
+    *taken = true;
+    const Plan p = make_plan(calls, n, 4);
+    const auto* x = static_cast<const uint16_t*>(calls[0].x);
+#define MI_Q4F(KT)                                                                                   \
+    case KT:                                                                                         \
+        if (p.pipe) {                                                                                \
+            constexpr int kRB = group_size(WK_Q4, KT, 4);                                            \
+            hipLaunchKernelGGL((gemv_q4_fast<KT, EPI, true, kRB>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+        } else {                                                                                     \
+            hipLaunchKernelGGL((gemv_q4_fast<KT, EPI, false, 1>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+        }                                                                                            \
+        break;
+    switch (K) {
+        MI_Q4F(576)
+        MI_Q4F(896)
+        MI_Q4F(1024)
+        MI_Q4F(1536)
+        default: *taken = false; return true;
+    }
+#undef MI_Q4F
+    return MI_HIP_OK(hipGetLastError());
+}
+
 template <int KIND, int EPI>
 bool launch_kind(hipStream_t s, const GemvCall* calls, int n, int vl) {
     if constexpr (KIND != WK_F16) {
@@ -636,6 +809,11 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
     const GemvCall& c = calls[0];
     const int vl = pick_vl(c.kind, c.M, rows, c.K);
     const bool add = c.epi == EPI_ADD;
+    if (c.kind == WK_Q4 && vl == 4 && gemv_mode() == 1) {
+        bool taken = false;
+        const bool ok = add ? launch_q4_fast<EPI_ADD>(s, calls, n, &taken) : launch_q4_fast<EPI_STORE>(s, calls, n, &taken);
+        if (taken) return ok;
+    }
     switch (c.kind) {
         case WK_F16: return add ? launch_kind<WK_F16, EPI_ADD>(s, calls, n, vl) : launch_kind<WK_F16, EPI_STORE>(s, calls, n, vl);
         case WK_I8:  return add ? launch_kind<WK_I8, EPI_ADD>(s, calls, n, vl) : launch_kind<WK_I8, EPI_STORE>(s, calls, n, vl);

@@ -13,6 +13,7 @@ namespace {
 DeviceInfo g_dev;
 bool g_inited = false;
 int g_gemm_mode = 0;
+int g_gemv_mode = 1;
 
 // Side table W pointer -> {kind, scale, N, K}; the counterpart of s_int8_aux / s_q4_aux
 // (LF/src/utils.cpp:194-231).  The reference is single threaded and takes no lock; a
@@ -57,6 +58,7 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 }  // namespace
 
 const DeviceInfo& device_info() { return g_dev; }
+int gemv_mode() { return g_gemv_mode; }
 
 }  // namespace mi
 
@@ -179,6 +181,7 @@ int mi_weight_kind(const void* W) {
 }
 
 void mi_set_gemm_mode(int mode) { g_gemm_mode = mode; }
+void mi_set_gemv_mode(int mode) { g_gemv_mode = mode; }
 
 // ---- hot path --------------------------------------------------------------------
 

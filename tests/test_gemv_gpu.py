@@ -22,9 +22,11 @@ SHAPES_Q4 = [(4864, 896), (896, 4864), (128, 896), (4608, 1024), (1024, 4608), (
 @pytest.fixture(scope="module")
 def queue():
     assert mil.lib().mi_init(0) == 1, "no gfx950 device"
+    mil.lib().mi_set_gemv_mode(0)          # reference evaluation order for every kind (bit-exact)
     q = mil.Queue()
     yield q
     q.finish()
+    mil.lib().mi_set_gemv_mode(1)
 
 
 def _run_linear(queue, M, N, K, x, W_host, scale_host=None, kind="f16", canary=True):

@@ -1,0 +1,93 @@
+"""Throughput variant of the Q4 GEMV (mi_set_gemv_mode(1), the default): same fp32 products as
+the reference kernel, summed in another order.  Bar: the stated tolerance (max-abs/rel 1e-3,
+cosine >= 0.9999) against the oracle, bit-exact wherever the arithmetic is exact (integer
+data, unit vectors), and bit-exact unpack indexing over all byte values."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from helpers import assert_tolerance, mil, synth_w, synth_x
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def queue():
+    assert mil.lib().mi_init(0) == 1, "no gfx950 device"
+    mil.lib().mi_set_gemv_mode(1)
+    q = mil.Queue()
+    yield q
+    q.finish()
+
+
+def _run(queue, N, K, x, p, sc, add_to=None):
+    xb, pb, sb = mil.Buffer.from_host(x), mil.Buffer.from_host(p), mil.Buffer.from_host(sc)
+    assert mil.nnopt_register_q4_weight(pb, sb, N, K)
+    pad = 64
+    guard = np.full(N + 2 * pad, 0x7BCD, np.uint16)
+    if add_to is not None:
+        guard[pad:-pad] = add_to.view(np.uint16)
+    ob = mil.Buffer.from_host(guard)
+    if add_to is None:
+        assert mil.pytorch_linear(queue, 1, N, K, xb, pb, ob.ptr + 2 * pad)
+    else:
+        assert mil.pytorch_linear_add(queue, 1, N, K, xb, pb, ob.ptr + 2 * pad)
+    queue.finish()
+    full = ob.read(np.uint16, guard.shape)
+    assert np.all(full[:pad] == 0x7BCD) and np.all(full[-pad:] == 0x7BCD)
+    mil.nnopt_unregister_weight(pb)
+    return full[pad:-pad]
+
+
+@pytest.mark.parametrize("N,K", [(4864, 896), (151936, 896), (4608, 1024), (8192, 576), (4100, 1536), (4099, 896)])
+def test_fast_q4_within_tolerance(queue, N, K):
+    print(f"fast q4 N={N} K={K}", flush=True)
+    W, x = synth_w(1000 + N, N, K), synth_x(1100 + K, K)
+    p, sc = mil.quantize_q4(W)
+    got = _run(queue, N, K, x, p, sc)
+    want = O.gemv_q4(x, p, sc.view(np.uint16))
+    assert_tolerance(got.view(np.float16), want.view(np.float16))
+    assert np.mean(got == want) > 0.97          # nearly all outputs are the same half
+
+
+def test_fast_q4_exact_on_integer_data_and_all_bytes(queue):
+    # integer activations and power-of-two scales: every order of the fp32 sum is exact
+    rng = np.random.default_rng(5)
+    N, K = 4096, 896
+    p = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
+    p[0, :256] = np.arange(256, dtype=np.uint8)
+    sc = (2.0 ** rng.integers(-8, -3, (N, K // 32))).astype(np.float16)
+    x = rng.integers(-4, 5, K).astype(np.float16)
+    got = _run(queue, N, K, x, p, sc)
+    nib = np.stack([p & 15, p >> 4], -1).reshape(N, K).astype(np.int64) - 8
+    want = ((nib * np.repeat(sc.astype(np.float64), 32, axis=1)) @ x.astype(np.float64)).astype(np.float16)
+    assert np.array_equal(got.view(np.float16), want)
+    assert np.array_equal(got, O.gemv_q4(x, p, sc.view(np.uint16)))
+
+
+def test_fast_q4_unit_vectors_and_subnormal_activations(queue):
+    N, K = 4096, 896
+    W = synth_w(1200, N, K)
+    p, sc = mil.quantize_q4(W)
+    nib = np.stack([p & 15, p >> 4], -1).reshape(N, K).astype(np.float32) - 8
+    for k in (0, 1, 4, 5, 31, 32, 511, 512, 895):
+        x = np.zeros(K, np.float16)
+        x[k] = 1.0
+        want = (nib[:, k] * sc[:, k // 32].astype(np.float32)).astype(np.float16)
+        assert np.array_equal(_run(queue, N, K, x, p, sc).view(np.float16), want), k
+    x = synth_x(1201, K)
+    x[::5] = np.float16(6e-8)
+    x[1::5] = np.float16(-2e-5)
+    got = _run(queue, N, K, x, p, sc)
+    assert_tolerance(got.view(np.float16), O.gemv_q4(x, p, sc.view(np.uint16)).view(np.float16))
+
+
+def test_fast_q4_residual_epilogue(queue):
+    N, K = 8192, 896
+    W, x = synth_w(1300, N, K), synth_x(1301, K)
+    res0 = synth_x(1302, N)
+    p, sc = mil.quantize_q4(W)
+    got = _run(queue, N, K, x, p, sc, add_to=res0)
+    want = res0.view(np.uint16).copy()
+    O.lib.orc_gemv_q4_add(O.u16(x), p, np.ascontiguousarray(sc.view(np.uint16)), want, N, K)
+    assert_tolerance(got.view(np.float16), want.view(np.float16))
