@@ -230,6 +230,59 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     const int m = blockIdx.y;
     x += static_cast<size_t>(m) * KT;
 
+    // One row batch in registers: weights, scales and (EPI_ADD) the residual, all fetched
+    // together so that the epilogue never waits on a late load.  Addresses are a per-batch
+    // scalar base plus a per-lane offset that never changes, so a fetch costs no vector
+    // arithmetic beyond one select for rows past N (those re-read the batch's first row).
+    struct Batch {
+        uint32_t w[NIT][WD];
+        uint16_t s[KIND == WK_Q4 ? NIT : 1];
+        uint16_t res;
+        uint16_t* ybase;    // &y[m][first row of the batch], uniform
+        int yoff;           // row inside the batch, -1 when the lane's row is past N
+    };
+    const uint32_t lane_w = r * ROWB + koff / T::EPV * T::BPV;     // byte offset of the lane's weights
+    const uint32_t lane_w0 = koff / T::EPV * T::BPV;               // same column, first row of the batch
+    auto fetch = [&](Batch& b, int rb) {
+        const Seg sg = L.nseg == 1 ? L.s[0] : find_segment(L, rb);
+        const int row0 = (rb - sg.first) * RPW;
+        const bool valid = row0 + r < sg.N;
+        const int rr = valid ? r : 0;
+        const uint8_t* wb = sg.W + static_cast<size_t>(row0) * ROWB;
+        const uint32_t wo = valid ? lane_w : lane_w0;
+        b.ybase = sg.y + static_cast<size_t>(m) * sg.N + row0;
+        b.yoff = valid ? r : -1;
+        if constexpr (KIND == WK_I8) b.s[0] = (sg.sc + row0)[rr];
+        if constexpr (EPI == EPI_ADD) b.res = b.ybase[rr];
+        #pragma unroll
+        for (int j = 0; j < NIT; ++j) {
+            // lanes idle in a partial last iteration re-read the start of their row, so that
+            // every lane issues the same number of loads (the value is never used)
+            const bool active = j * EIT + koff < KT;
+            load_dwords<WD, true>(b.w[j], wb + (active ? wo + j * ITB : wo - lane_w0));
+            if constexpr (KIND == WK_Q4)
+                b.s[j] = (sg.sc + static_cast<size_t>(row0) * (KT / 32))[rr * (KT / 32) + (active ? j * 16 + (g * VL) / 4 : 0)];
+        }
+    };
+    // Order of issue: the first group of row batches, then the activations: both are in
+    // flight before anything waits.
+    const int nw = gridDim.x * kWavesPerBlock;
+    int rb = blockIdx.x * kWavesPerBlock + wave;
+    if (rb >= L.nbatch) return;
+    constexpr int GB = PIPE ? RB : 1;
+    struct Group { Batch b[GB]; };
+    const int first = rb;
+    // A wavefront owns batches rb, rb + nw, rb + 2 nw, ...; it takes them GB at a time.  A batch
+    // index past the end is replaced by the wavefront's first batch (a cached re-read whose
+    // result is dropped), so every fetch issues the same loads.
+    auto fetch_group = [&](Group& gr, int at) {
+        #pragma unroll
+        for (int u = 0; u < GB; ++u) fetch(gr.b[u], at + u * nw < L.nbatch ? at + u * nw : first);
+    };
+    const int step = nw * GB;
+    Group g0, g1;
+    fetch_group(g0, rb);
+
     uint32_t xr[NIT][XD];
     #pragma unroll
     for (int j = 0; j < NIT; ++j) {
@@ -240,35 +293,6 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
         }
     }
 
-    // One row batch in registers: weights, scales and (EPI_ADD) the residual, all fetched
-    // together so that the epilogue never waits on a late load.
-    struct Batch {
-        uint32_t w[NIT][WD];
-        uint16_t s[KIND == WK_Q4 ? NIT : 1];
-        uint16_t res;
-        uint16_t* yrow;     // null when the lane's row is past N
-    };
-    auto fetch = [&](Batch& b, int rb) {
-        const Seg sg = find_segment(L, rb);
-        const int row = (rb - sg.first) * RPW + r;
-        const bool valid = row < sg.N;
-        const int rowc = valid ? row : sg.N - 1;
-        uint16_t* yp = sg.y + static_cast<size_t>(m) * sg.N + rowc;
-        b.yrow = valid ? yp : nullptr;
-        if constexpr (KIND == WK_I8) b.s[0] = sg.sc[rowc];
-        if constexpr (EPI == EPI_ADD) b.res = *yp;
-        const uint8_t* wrow = sg.W + static_cast<size_t>(rowc) * ROWB;
-        const int lane_off = koff / T::EPV * T::BPV;
-        #pragma unroll
-        for (int j = 0; j < NIT; ++j) {
-            // lanes idle in a partial last iteration re-read the start of the row, so that
-            // every lane issues the same number of loads (the value is never used)
-            const bool active = j * EIT + koff < KT;
-            load_dwords<WD, true>(b.w[j], wrow + (active ? j * ITB + lane_off : 0));
-            if constexpr (KIND == WK_Q4)
-                b.s[j] = sg.sc[static_cast<size_t>(rowc) * (KT / 32) + (active ? j * 16 + (g * VL) / 4 : 0)];
-        }
-    };
     auto consume = [&](const Batch& b) {
         float acc[VL];
         #pragma unroll
@@ -283,7 +307,7 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
             }
         }
         const float sum = reduce_row<VL>(acc);
-        if (g == 0 && b.yrow) {
+        if (g == 0 && b.yoff >= 0) {
             float out;
             if constexpr (KIND == WK_I8) {
                 const float s = h_f(b.s[0]);
@@ -291,37 +315,23 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
             } else {
                 out = EPI == EPI_ADD ? sum + h_f(b.res) : sum;
             }
-            *b.yrow = f_h(out);
+            b.ybase[b.yoff] = f_h(out);
         }
     };
 
-    const int nw = gridDim.x * kWavesPerBlock;
-    int rb = blockIdx.x * kWavesPerBlock + wave;
-    if (rb >= L.nbatch) return;
+    auto consume_group = [&](const Group& gr, int at) {
+        #pragma unroll
+        for (int u = 0; u < GB; ++u)
+            if (at + u * nw < L.nbatch) consume(gr.b[u]);
+    };
     if constexpr (!PIPE) {
-        for (; rb < L.nbatch; rb += nw) {
-            Batch b;
-            fetch(b, rb);
-            consume(b);
+        while (true) {
+            consume_group(g0, rb);
+            rb += step;
+            if (rb >= L.nbatch) break;
+            fetch_group(g0, rb);
         }
     } else {
-        // A wavefront owns batches rb, rb + nw, rb + 2 nw, ...; it takes them RB at a time.
-        // A batch index past the end is replaced by the wavefront's first batch (a cached
-        // re-read whose result is dropped), so every fetch issues the same loads.
-        struct Group { Batch b[RB]; };
-        const int first = rb;
-        auto fetch_group = [&](Group& gr, int at) {
-            #pragma unroll
-            for (int u = 0; u < RB; ++u) fetch(gr.b[u], at + u * nw < L.nbatch ? at + u * nw : first);
-        };
-        auto consume_group = [&](const Group& gr, int at) {
-            #pragma unroll
-            for (int u = 0; u < RB; ++u)
-                if (at + u * nw < L.nbatch) consume(gr.b[u]);
-        };
-        const int step = nw * RB;
-        Group g0, g1;
-        fetch_group(g0, rb);
         while (true) {
             fetch_group(g1, rb + step);
             consume_group(g0, rb);
@@ -363,53 +373,75 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
     const int m = blockIdx.y;
     x += static_cast<size_t>(m) * KT;
 
-    // xp[j][4 d + i]: activations paired for dword d of the lane's 16 weight bytes:
-    // i = 0: (x0, x4), 1: (x1, x5), 2: (x2, x6), 3: (x3, x7) of elements 8 d .. 8 d + 7.
-    uint32_t xp[NIT][16];
-    float m8sx[NIT];                                    // -8 * sum of the block's activations
-    #pragma unroll
-    for (int j = 0; j < NIT; ++j) {
-        uint32_t raw[16];
-        if (j * EIT + koff < KT) load_dwords<16, false>(raw, x + j * EIT + koff);
-        else {
-            #pragma unroll
-            for (int i = 0; i < 16; ++i) raw[i] = 0u;
-        }
-        float sx = 0.0f;
-        #pragma unroll
-        for (int i = 0; i < 16; ++i) sx += lo_f(raw[i]) + hi_f(raw[i]);
-        m8sx[j] = -8.0f * sx;
-        #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            xp[j][4 * d + 0] = __builtin_amdgcn_perm(raw[4 * d + 2], raw[4 * d + 0], 0x05040100u);
-            xp[j][4 * d + 1] = __builtin_amdgcn_perm(raw[4 * d + 2], raw[4 * d + 0], 0x07060302u);
-            xp[j][4 * d + 2] = __builtin_amdgcn_perm(raw[4 * d + 3], raw[4 * d + 1], 0x05040100u);
-            xp[j][4 * d + 3] = __builtin_amdgcn_perm(raw[4 * d + 3], raw[4 * d + 1], 0x07060302u);
-        }
-    }
-
     struct Batch {
         uint32_t w[NIT][4];
         uint16_t s[NIT];
         uint16_t res;
-        uint16_t* yrow;
+        uint16_t* ybase;    // &y[m][first row of the batch], uniform
+        int yoff;           // row inside the batch, -1 when the lane's row is past N
     };
+    const uint32_t lane_w = r * ROWB + g * 16, lane_w0 = g * 16;
     auto fetch = [&](Batch& b, int rb) {
-        const Seg sg = find_segment(L, rb);
-        const int row = (rb - sg.first) * 4 + r;
-        const bool valid = row < sg.N;
-        const int rowc = valid ? row : sg.N - 1;
-        uint16_t* yp = sg.y + static_cast<size_t>(m) * sg.N + rowc;
-        b.yrow = valid ? yp : nullptr;
-        if constexpr (EPI == EPI_ADD) b.res = *yp;
-        const uint8_t* wrow = sg.W + static_cast<size_t>(rowc) * ROWB;
+        const Seg sg = L.nseg == 1 ? L.s[0] : find_segment(L, rb);
+        const int row0 = (rb - sg.first) * 4;
+        const bool valid = row0 + r < sg.N;
+        const int rr = valid ? r : 0;
+        const uint8_t* wb = sg.W + static_cast<size_t>(row0) * ROWB;
+        const uint16_t* sb = sg.sc + static_cast<size_t>(row0) * (KT / 32);
+        const uint32_t wo = valid ? lane_w : lane_w0;
+        b.ybase = sg.y + static_cast<size_t>(m) * sg.N + row0;
+        b.yoff = valid ? r : -1;
+        if constexpr (EPI == EPI_ADD) b.res = b.ybase[rr];
         #pragma unroll
         for (int j = 0; j < NIT; ++j) {
             const bool active = j * EIT + koff < KT;
-            load_dwords<4, true>(b.w[j], wrow + (active ? j * 256 + g * 16 : 0));
-            b.s[j] = sg.sc[static_cast<size_t>(rowc) * (KT / 32) + (active ? j * 16 + g : 0)];
+            load_dwords<4, true>(b.w[j], wb + (active ? wo + j * 256 : wo - lane_w0));
+            b.s[j] = sb[rr * (KT / 32) + (active ? j * 16 + g : 0)];
         }
     };
+    // The first weights are requested before the activations: the pairing of x below waits
+    // for x to arrive, and that wait should not delay the first fetch by a memory latency.
+    const int nw = gridDim.x * kWavesPerBlock;
+    int rb = blockIdx.x * kWavesPerBlock + wave;
+    if (rb >= L.nbatch) return;
+    struct Group { Batch b[PIPE ? RB : 1]; };
+    constexpr int GB = PIPE ? RB : 1;
+    const int first = rb;
+    auto fetch_group = [&](Group& gr, int at) {
+        #pragma unroll
+        for (int u = 0; u < GB; ++u) fetch(gr.b[u], at + u * nw < L.nbatch ? at + u * nw : first);
+    };
+    Group g0, g1;
+    fetch_group(g0, rb);
+
+    // xp[j][4 d + i]: activations paired for dword d of the lane's 16 weight bytes:
+    // i = 0: (x0, x4), 1: (x1, x5), 2: (x2, x6), 3: (x3, x7) of elements 8 d .. 8 d + 7.
+    uint32_t xp[NIT][16];
+    float m8sx[NIT];                                    // -8 * sum of the block's activations
+    uint32_t raw[NIT][16];
+    #pragma unroll
+    for (int j = 0; j < NIT; ++j) {
+        if (j * EIT + koff < KT) load_dwords<16, false>(raw[j], x + j * EIT + koff);
+        else {
+            #pragma unroll
+            for (int i = 0; i < 16; ++i) raw[j][i] = 0u;
+        }
+    }
+    #pragma unroll
+    for (int j = 0; j < NIT; ++j) {
+        float sx = 0.0f;
+        #pragma unroll
+        for (int i = 0; i < 16; ++i) sx += lo_f(raw[j][i]) + hi_f(raw[j][i]);
+        m8sx[j] = -8.0f * sx;
+        #pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            xp[j][4 * d + 0] = __builtin_amdgcn_perm(raw[j][4 * d + 2], raw[j][4 * d + 0], 0x05040100u);
+            xp[j][4 * d + 1] = __builtin_amdgcn_perm(raw[j][4 * d + 2], raw[j][4 * d + 0], 0x07060302u);
+            xp[j][4 * d + 2] = __builtin_amdgcn_perm(raw[j][4 * d + 3], raw[j][4 * d + 1], 0x05040100u);
+            xp[j][4 * d + 3] = __builtin_amdgcn_perm(raw[j][4 * d + 3], raw[j][4 * d + 1], 0x07060302u);
+        }
+    }
+
     auto consume = [&](const Batch& b) {
         float acc = 0.0f;
         #pragma unroll
@@ -437,36 +469,26 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
         acc = add_from_above<4>(acc);
         acc = add_from_above<2>(acc);
         acc = add_from_above<1>(acc);
-        if (g == 0 && b.yrow) {
+        if (g == 0 && b.yoff >= 0) {
             const float out = EPI == EPI_ADD ? acc + h_f(b.res) : acc;
-            *b.yrow = f_h(out);
+            b.ybase[b.yoff] = f_h(out);
         }
     };
 
-    const int nw = gridDim.x * kWavesPerBlock;
-    int rb = blockIdx.x * kWavesPerBlock + wave;
-    if (rb >= L.nbatch) return;
+    auto consume_group = [&](const Group& gr, int at) {
+        #pragma unroll
+        for (int u = 0; u < GB; ++u)
+            if (at + u * nw < L.nbatch) consume(gr.b[u]);
+    };
+    const int step = nw * GB;
     if constexpr (!PIPE) {
-        for (; rb < L.nbatch; rb += nw) {
-            Batch b;
-            fetch(b, rb);
-            consume(b);
+        while (true) {
+            consume_group(g0, rb);
+            rb += step;
+            if (rb >= L.nbatch) break;
+            fetch_group(g0, rb);
         }
     } else {
-        struct Group { Batch b[RB]; };
-        const int first = rb;
-        auto fetch_group = [&](Group& gr, int at) {
-            #pragma unroll
-            for (int u = 0; u < RB; ++u) fetch(gr.b[u], at + u * nw < L.nbatch ? at + u * nw : first);
-        };
-        auto consume_group = [&](const Group& gr, int at) {
-            #pragma unroll
-            for (int u = 0; u < RB; ++u)
-                if (at + u * nw < L.nbatch) consume(gr.b[u]);
-        };
-        const int step = nw * RB;
-        Group g0, g1;
-        fetch_group(g0, rb);
         while (true) {
             fetch_group(g1, rb + step);
             consume_group(g0, rb);
