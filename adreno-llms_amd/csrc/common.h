@@ -33,6 +33,7 @@ const DeviceInfo& device_info();
 // 0 = every GEMV evaluates the reference kernels' sum in their order (bit-exact);
 // 1 = Q4 may use the throughput kernel (same fp32 sum, other order).
 int gemv_mode();
+int gemm_mode();   // 0 auto, 1 batched GEMV, 2 / 3 force the 64 x 64 / 128 x 128 MFMA tile
 
 // M rows of x (stride K) against one W; y rows have stride N.
 struct GemvCall {

@@ -59,6 +59,7 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
 const DeviceInfo& device_info() { return g_dev; }
 int gemv_mode() { return g_gemv_mode; }
+int gemm_mode() { return g_gemm_mode; }
 
 }  // namespace mi
 
@@ -195,7 +196,7 @@ int mi_linear(void* stream, int M, int N, int K, const void* x, const void* W, v
     if (!resolve("mi_linear", W, N, K, &e)) return 0;
     // M > 1: a real contraction goes to the MFMA GEMM; small batches, and every batch in
     // mode 1, run the GEMV once per row of x, as the reference's quantised prefill does.
-    if (M >= 16 && g_gemm_mode == 0 && gemm_supported(e.kind, M, N, K))
+    if (M >= 16 && g_gemm_mode != 1 && gemm_supported(e.kind, M, N, K))
         return launch_gemm(as_stream(stream), e.kind, M, N, K, x, W, e.scale, out) ? 1 : 0;
     GemvCall c;
     c.x = x; c.W = W; c.scale = e.scale; c.y = out;

@@ -33,7 +33,9 @@ def _ulp_apart(a_u16, b_u16):
     return np.abs(a - b) / step
 
 
-def _gemm(queue, M, N, K, X, W_host, scale_host, kind):
+def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0):
+    """tile is the mi_set_gemm_mode value: 0 = the library's own choice, 1 = rows of GEMV,
+    2 / 3 = the 64 x 64 / 128 x 128 MFMA kernel."""
     xb, wb = mil.Buffer.from_host(X), mil.Buffer.from_host(W_host)
     sb = mil.Buffer.from_host(scale_host) if scale_host is not None else None
     if kind == "i8":
@@ -41,21 +43,26 @@ def _gemm(queue, M, N, K, X, W_host, scale_host, kind):
     pad = 128
     guard = np.full(M * N + 2 * pad, 0x7BCD, np.uint16)
     ob = mil.Buffer.from_host(guard)
-    assert mil.pytorch_linear(queue, M, N, K, xb, wb, ob.ptr + 2 * pad)
-    queue.finish()
+    mil.lib().mi_set_gemm_mode(tile)
+    try:
+        assert mil.pytorch_linear(queue, M, N, K, xb, wb, ob.ptr + 2 * pad)
+        queue.finish()
+    finally:
+        mil.lib().mi_set_gemm_mode(0)
     full = ob.read(np.uint16, guard.shape)
     assert np.all(full[:pad] == 0x7BCD) and np.all(full[-pad:] == 0x7BCD), "wrote outside out[M,N]"
     mil.nnopt_unregister_weight(wb)
     return full[pad:-pad].reshape(M, N)
 
 
+@pytest.mark.parametrize("tile", [2, 3])
 @pytest.mark.parametrize("M", [16, 64, 100, 512])
-@pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (200, 128), (130, 576)])
-def test_int8_gemm_matches_rows_of_gemv(queue, M, N, K):
-    print(f"int8 gemm M={M} N={N} K={K}", flush=True)
+@pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (200, 128), (130, 576), (131, 64)])
+def test_int8_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
+    print(f"int8 gemm M={M} N={N} K={K} tile mode {tile}", flush=True)
     W, X = synth_w(700 + N, N, K), synth_x(800 + M, M, K)
     q, s = mil.quantize_int8(W)
-    got = _gemm(queue, M, N, K, X, q, s, "i8")
+    got = _gemm(queue, M, N, K, X, q, s, "i8", tile)
     want = O.gemm_i8(X, q, s.view(np.uint16))
     assert_tolerance(got.view(np.float16), want.view(np.float16))
     d = _ulp_apart(got, want)
@@ -63,29 +70,33 @@ def test_int8_gemm_matches_rows_of_gemv(queue, M, N, K):
     assert np.mean(got == want) > 0.99
 
 
-@pytest.mark.parametrize("M,N,K", [(64, 4864, 896), (256, 896, 4864), (33, 200, 128)])
-def test_fp16_gemm_matches_rows_of_gemv(queue, M, N, K):
+@pytest.mark.parametrize("tile", [2, 3])
+@pytest.mark.parametrize("M,N,K", [(64, 4864, 896), (256, 896, 4864), (33, 200, 128), (130, 131, 64)])
+def test_fp16_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
+    print(f"fp16 gemm M={M} N={N} K={K} tile mode {tile}", flush=True)
     W, X = synth_w(900 + N, N, K), synth_x(901 + M, M, K)
-    got = _gemm(queue, M, N, K, X, W, None, "f16")
+    got = _gemm(queue, M, N, K, X, W, None, "f16", tile)
     want = O.gemm_f16(X, W)
     assert_tolerance(got.view(np.float16), want.view(np.float16))
     assert _ulp_apart(got, want).max() <= 1
 
 
-def test_gemm_exact_on_integer_data(queue):
+@pytest.mark.parametrize("tile", [2, 3])
+def test_gemm_exact_on_integer_data(queue, tile):
     # small integers: every partial sum is exact in fp32, so any summation order gives the same bits
     rng = np.random.default_rng(3)
     M, N, K = 96, 192, 256
     q = rng.integers(-127, 128, (N, K)).astype(np.int8)
     X = rng.integers(-3, 4, (M, K)).astype(np.float16)
     s = (2.0 ** rng.integers(-10, -6, N)).astype(np.float16)
-    got = _gemm(queue, M, N, K, X, q, s, "i8")
+    got = _gemm(queue, M, N, K, X, q, s, "i8", tile)
     want = ((X.astype(np.int64) @ q.astype(np.int64).T).astype(np.float64) * s.astype(np.float64)).astype(np.float16)
     assert np.array_equal(got.view(np.float16), want)
     assert np.array_equal(got, O.gemm_i8(X, q, s.view(np.uint16)))
 
 
-def test_gemm_unit_rows_pick_weight_columns(queue):
+@pytest.mark.parametrize("tile", [2, 3])
+def test_gemm_unit_rows_pick_weight_columns(queue, tile):
     # x rows are unit vectors: out[i, :] must be the dequantised column k_i of W (index check)
     M, N, K = 64, 320, 896
     W = synth_w(910, N, K)
@@ -93,7 +104,7 @@ def test_gemm_unit_rows_pick_weight_columns(queue):
     ks = (np.arange(M) * 37 + 5) % K
     X = np.zeros((M, K), np.float16)
     X[np.arange(M), ks] = 1.0
-    got = _gemm(queue, M, N, K, X, q, s, "i8").view(np.float16)
+    got = _gemm(queue, M, N, K, X, q, s, "i8", tile).view(np.float16)
     want = (q[:, ks].T.astype(np.float32) * s.astype(np.float32)[None, :]).astype(np.float16)
     assert np.array_equal(got, want)
 
@@ -120,9 +131,5 @@ def test_batched_gemv_mode_stays_bit_exact(queue):
     M, N, K = 32, 896, 896
     W, X = synth_w(930, N, K), synth_x(931, M, K)
     q, s = mil.quantize_int8(W)
-    mil.lib().mi_set_gemm_mode(1)
-    try:
-        got = _gemm(queue, M, N, K, X, q, s, "i8")
-    finally:
-        mil.lib().mi_set_gemm_mode(0)
+    got = _gemm(queue, M, N, K, X, q, s, "i8", tile=1)
     assert np.array_equal(got, O.gemm_i8(X, q, s.view(np.uint16)))
