@@ -15,6 +15,8 @@
 // accumulators of 32 x 32.
 #include "common.h"
 #include <hip/hip_fp16.h>
+#include <type_traits>
+#include <utility>
 
 namespace mi {
 namespace {
@@ -179,179 +181,368 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const uint16_t* __restri
     }
 }
 
-// ---- 128 x 128 tile, two wavefronts ------------------------------------------------
+// ---- int8 weights, wide tiles fed by direct global -> LDS loads ------------------------
 //
-// The kernel above spends more LDS bandwidth than matrix-core time: a wavefront that owns
-// 64 x 64 outputs reads four operand fragments for four MFMAs.  Here a block is 128 (rows of
-// x) x 128 (rows of W) with only two wavefronts, each owning all 128 rows of x against 64
-// rows of W: six fragments for eight MFMAs, and accumulators of 128 registers per lane.
-// Four such blocks share a CU (K-tile 32, two LDS stages of 20 KB each), i.e. two wavefronts
-// per SIMD.  W is the MFMA "A" operand and x the "B" operand, so a lane ends up with four
-// consecutive output columns of one output row: the epilogue scales them and writes 8 bytes
-// per lane instead of four 2-byte stores.
-constexpr int kKT2 = 32;
-constexpr int kLd2 = kKT2 + 8;     // 40 halves = 80 bytes: 8 consecutive rows, 8 different 16-byte slots
+// What bounds the kernel above is the rate at which a CU can fill LDS (about 150 bytes/ns,
+// against 530 bytes/ns for reads and one 32x32x16 MFMA per 15.6 ns per SIMD) and the fragment
+// reads that are not overlapped with the MFMAs of the same wavefront.  This kernel therefore
+//  * keeps W as int8 in LDS (half the fill bytes) and converts a fragment to fp16 in registers
+//    after reading it; the four wavefronts of a block own disjoint rows of W (64 each, so the
+//    block covers 256 rows of W) and share the 32*TM rows of x, so no fragment of W is
+//    converted twice;
+//  * fills LDS with global_load_lds_dwordx4 (no registers, no ds_write), four to eight stages of K = 64;
+//    16-byte chunks are XOR-swizzled inside a row so that fragment reads are conflict-free
+//    without padding (a wavefront's load always fills 1 KB of consecutive LDS);
+//  * reads the fragments of the next 32 values of K before issuing the MFMAs of the current
+//    ones, with one barrier per stage placed in the middle of a stage, where the data of the
+//    next stage is known to have landed;
+//  * orders K inside a group of 32 so that a lane's 16 consecutive int8 feed two MFMAs: lanes
+//    0-31 supply k = 0..7 then 8..15, lanes 32-63 supply 16..23 then 24..31, for W and x alike.
+// W is the MFMA "A" operand and x the "B" operand, so a lane ends up with four consecutive
+// output columns of one output row and stores them as 8 bytes.
+namespace wide {
 
-template <int KIND>
-__global__ __launch_bounds__(128) void gemm_kernel_128x128(const uint16_t* __restrict__ X,
-                                                          const uint8_t* __restrict__ W,
-                                                          const uint16_t* __restrict__ scale,
-                                                          uint16_t* __restrict__ out, int M, int N, int K) {
-    constexpr int BM = 128, BN = 128, NT = 128;
-    constexpr int TM = 4, TN = 2;                                       // 32-wide tiles per wavefront
-    constexpr int A_CHUNKS = BM * (kKT2 / 8) / NT;                      // 4: 16-byte chunks of x per thread
-    constexpr int B_BYTES = KIND == WK_I8 ? 1 : 2;
-    constexpr int B_CPR = kKT2 * B_BYTES / 16;                          // chunks per W row: 2 (int8) or 4
-    constexpr int B_CHUNKS = BN * B_CPR / NT;                           // 2 or 4
-    constexpr int kStage = (BM + BN) * kLd2;                            // halves per LDS stage
+constexpr int kBN = 256;                    // rows of W per block
+// LDS stages (K = 64 each) for 32 * tm rows of x: as many as 160 KB hold, at most 8.  A stage is
+// requested stages - 2 stage times before it is needed, which is what covers the load latency.
+constexpr int stages_for(int tm) { return tm >= 4 ? 4 : tm == 3 ? 5 : tm == 2 ? 6 : 8; }
+constexpr int kWStage = kBN * 64;           // bytes of W (int8) per stage
+typedef __attribute__((address_space(3))) uint8_t lds_u8;
+typedef __attribute__((address_space(1))) const uint8_t glb_u8;
 
-    __shared__ __attribute__((aligned(16))) uint16_t lds[2 * kStage];
+__device__ __forceinline__ void lds_fill16(const uint8_t* g, uint8_t* l) {
+    __builtin_amdgcn_global_load_lds((glb_u8*)g, (lds_u8*)l, 16, 0, 0);   // address-space casts
+}
+#define MI_LDS_READ16(dst, addr, imm) \
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(imm))
+#define MI_WAIT_LGKM(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n) : "memory")
+#define MI_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
+#define MI_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-    const int tid = threadIdx.x, lane = tid % 64, wn = tid / 64;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    const int gk = lane / 32, li = lane % 32;
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): indices are compile-time
+// constants inside f (immediate operands, register array subscripts)
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
 
-    floatx16 acc[TN][TM];
+template <int TM>
+struct Frags {
+    u32x4 w[2];          // 16 int8 of two 32-row fragments of W, as read from LDS
+    uint32_t wf[2][2][4];  // the same as fp16: [fragment][MFMA of the pair][4 dwords = 8 halves]
+    u32x4 x[2][TM];      // [MFMA of the pair][32-row fragment of x], 8 halves each
+};
+
+template <int TM>
+__global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__ X,
+                                                   const uint8_t* __restrict__ W,
+                                                   const uint16_t* __restrict__ scale,
+                                                   uint16_t* __restrict__ out, int M, int N, int K) {
+    constexpr int BM = 32 * TM;
+    constexpr int kXStage = BM * 128;                    // bytes of x (fp16) per stage
+    constexpr int kStage = kXStage + kWStage;
+    constexpr int kLoads = TM + 4;                       // global -> LDS loads per wavefront and stage
+    constexpr int kStages = stages_for(TM);
+    constexpr int kReads = 2 + 2 * TM;                   // LDS reads per set of fragments
+    constexpr int kMfmas = 4 * TM;                       // MFMAs per half stage (K = 32)
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane >> 5, li = lane & 31;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * kBN;
+    const uint32_t lbase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_u8*)lds));
+
+    // per-row scales of this lane's output columns, requested before anything else so that they
+    // are in registers long before the epilogue: sc[u][rq] = 4 fp16 scales of columns nq .. nq + 3
+    const bool cols4 = (N % 4) == 0 && reinterpret_cast<uintptr_t>(scale) % 8 == 0;
+    uint2 sc[2][4];
     #pragma unroll
-    for (int u = 0; u < TN; ++u)
+    for (int u = 0; u < 2; ++u) {
+        #pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+            const int nq = n0 + 64 * w + 32 * u + 8 * rq + 4 * g;
+            if (cols4 && nq + 3 < N) {
+                sc[u][rq] = *reinterpret_cast<const uint2*>(scale + nq);
+            } else {
+                uint32_t h[4];
+                #pragma unroll
+                for (int e = 0; e < 4; ++e) h[e] = scale[nq + e < N ? nq + e : N - 1];
+                sc[u][rq] = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+            }
+        }
+    }
+
+    // --- fill side: lane i of load j writes LDS bytes [1024 j + 16 i, +16) of its region --------
+    // x: load j covers rows 8j..8j+7 (128 bytes each, 8 chunks); slot p of row r holds chunk p ^ ((r >> 1) & 7)
+    // W: load j covers rows 16j..16j+15 (64 bytes each, 4 chunks); slot p of row r holds chunk p ^ ((r >> 2) & 3)
+    uint32_t xsrc[TM], wsrc[4];
+    #pragma unroll
+    for (int jj = 0; jj < TM; ++jj) {
+        const int r = 8 * (w + 4 * jj) + (lane >> 3);
+        const int c = (lane & 7) ^ ((r >> 1) & 7);
+        const int m = m0 + r < M ? m0 + r : M - 1;
+        xsrc[jj] = static_cast<uint32_t>(m) * K * 2u + c * 16u;
+    }
+    #pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+        const int r = 16 * (4 * w + jj) + (lane >> 2);
+        const int c = (lane & 3) ^ ((r >> 2) & 3);
+        const int n = n0 + r < N ? n0 + r : N - 1;
+        wsrc[jj] = static_cast<uint32_t>(n) * K + c * 16u;
+    }
+    const uint8_t* Xb = reinterpret_cast<const uint8_t*>(X);
+    // load j (0 .. kLoads - 1) of this wavefront for K-stage stage_k into LDS slot `slot`
+    auto fill_one = [&](int stage_k, int slot, auto jc) {
+        constexpr int j = decltype(jc)::value;
+        uint8_t* xs = lds + slot * kStage;
+        if constexpr (j < TM)
+            lds_fill16(Xb + static_cast<size_t>(stage_k) * 128 + xsrc[j], xs + 1024 * (w + 4 * j));
+        else
+            lds_fill16(W + static_cast<size_t>(stage_k) * 64 + wsrc[j - TM], xs + kXStage + 1024 * (4 * w + (j - TM)));
+    };
+    auto fill_stage = [&](int stage_k, int slot) {
+        static_for<kLoads>([&](auto jc) { fill_one(stage_k, slot, jc); });
+    };
+
+    // --- read side -------------------------------------------------------------------------------
+    // pair S (0, 1) of a stage, MFMA e (0, 1) of the pair: x chunk 4S + 2g + e, W chunk 2S + g
+    const uint32_t xrow = lbase + li * 128u, xq = (2u * g) ^ ((li >> 1) & 7u);
+    const uint32_t wrow = lbase + kXStage + (64u * w + li) * 64u, wq = g ^ ((li >> 2) & 3u);
+    uint32_t xoff[2][2], woff[2];
+    #pragma unroll
+    for (int S = 0; S < 2; ++S) {
+        #pragma unroll
+        for (int e = 0; e < 2; ++e) xoff[S][e] = xrow + (((4u * S + e) ^ xq) << 4);
+        woff[S] = wrow + (((2u * S) ^ wq) << 4);
+    }
+    // LDS read j (0 .. kReads - 1) of a set: the two W fragments first, then x for the first and
+    // the second MFMA of the pair
+    auto read_one = [&](Frags<TM>& F, uint32_t slot_bytes, auto Sc, auto jc) {
+        constexpr int S = decltype(Sc)::value, j = decltype(jc)::value;
+        if constexpr (j < 2) {
+            const uint32_t a = woff[S] + slot_bytes;
+            MI_LDS_READ16(F.w[j], a, j * 32 * 64);
+        } else {
+            constexpr int e = (j - 2) / TM, t = (j - 2) % TM;
+            const uint32_t a = xoff[S][e] + slot_bytes;
+            MI_LDS_READ16(F.x[e][t], a, t * 4096);
+        }
+    };
+    // conversion j (0 .. 7) of a set: dword j % 4 of W fragment j / 4 becomes four halves
+    auto convert_one = [&](Frags<TM>& F, auto jc) {
+        constexpr int j = decltype(jc)::value, u = j / 4, d = j % 4;
+        i8x4_to_h4(F.w[u][d], F.wf[u][d / 2][2 * (d % 2)], F.wf[u][d / 2][2 * (d % 2) + 1]);
+    };
+
+    floatx16 acc[2][TM];
+    #pragma unroll
+    for (int u = 0; u < 2; ++u)
         #pragma unroll
         for (int t = 0; t < TM; ++t)
             #pragma unroll
             for (int r = 0; r < 16; ++r) acc[u][t][r] = 0.0f;
 
-    struct Regs { u32x4 a[A_CHUNKS]; u32x4 b[B_CHUNKS]; };
-    auto load_tile = [&](Regs& R, int k0) {
-        #pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) {
-            const int c = tid + i * NT, row = c / (kKT2 / 8), kc = c % (kKT2 / 8);
-            const int m = m0 + row < M ? m0 + row : M - 1;
-            R.a[i] = *reinterpret_cast<const u32x4*>(X + static_cast<size_t>(m) * K + k0 + kc * 8);
-        }
-        #pragma unroll
-        for (int i = 0; i < B_CHUNKS; ++i) {
-            const int c = tid + i * NT, row = c / B_CPR, kc = c % B_CPR;
-            const int n = n0 + row < N ? n0 + row : N - 1;
-            R.b[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
-                W + (static_cast<size_t>(n) * K + k0) * B_BYTES + kc * 16));
-        }
+    // MFMA n (0 .. kMfmas - 1) of a half stage; consecutive n use different accumulators
+    auto mfma_one = [&](const Frags<TM>& F, auto nc) {
+        constexpr int n = decltype(nc)::value, e = n / (2 * TM), u = (n / TM) % 2, t = n % TM;
+        const u32x4 wv = {F.wf[u][e][0], F.wf[u][e][1], F.wf[u][e][2], F.wf[u][e][3]};
+        acc[u][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, wv),
+                                                          __builtin_bit_cast(half8, F.x[e][t]), acc[u][t], 0, 0, 0);
     };
-    auto store_tile = [&](const Regs& R, uint16_t* Xs, uint16_t* Ws) {
+
+    // One half stage.  An MFMA keeps the matrix pipe busy for 32 cycles but issues in 4, and a
+    // wavefront issues in order: whatever else has to happen (LDS fills for a later stage, the
+    // LDS reads of the next fragments, their int8 -> fp16 conversion) is dealt out between the
+    // MFMAs, so that it runs in their shadow instead of draining the pipe.
+    //   C  = fragments being multiplied; Nx = fragments being prepared (LDS slot at next_bytes,
+    //   pair NS of that stage); FILL: also issue this wavefront's fills of stage fill_k.
+    auto half_stage = [&](Frags<TM>& C, Frags<TM>& Nx, uint32_t next_bytes, auto NSc, auto fillc,
+                          int fill_k, int fill_slot) {
+        constexpr bool FILL = decltype(fillc)::value;
+        constexpr int nF = FILL ? kLoads : 0;
+        constexpr int A = nF + kReads + 1 + 8;           // fills, reads, wait for W, conversions
+        static_for<kMfmas>([&](auto nc) {
+            constexpr int n = decltype(nc)::value;
+            mfma_one(C, nc);
+            MI_SCHED_FENCE();
+            constexpr int a0 = n * A / kMfmas, a1 = (n + 1) * A / kMfmas;
+            static_for<a1 - a0>([&](auto kc) {
+                constexpr int a = a0 + decltype(kc)::value;
+                if constexpr (a < nF) {
+                    fill_one(fill_k, fill_slot, std::integral_constant<int, a>{});
+                } else if constexpr (a < nF + kReads) {
+                    read_one(Nx, next_bytes, NSc, std::integral_constant<int, a - nF>{});
+                } else if constexpr (a == nF + kReads) {
+                    // LDS returns in order: the two W reads are back.  The registers are operands
+                    // of the wait so that the conversions that read them cannot be moved above it.
+                    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(Nx.w[0]), "+v"(Nx.w[1]) : "n"(kReads - 2) : "memory");
+                    MI_SCHED_FENCE();
+                } else {
+                    convert_one(Nx, std::integral_constant<int, a - nF - kReads - 1>{});
+                }
+            });
+            MI_SCHED_FENCE();
+        });
+        // The reads into Nx complete before this straight-line block ends: the compiler takes the
+        // asm outputs for ready values, so they must be, wherever it may place a register copy.
+        MI_WAIT_LGKM(0);
+        MI_SCHED_FENCE();
+    };
+
+    // waits until at most `stages` of this wavefront's stage fills are still in flight
+    auto wait_fills = [&](int stages) {
+        bool done = false;
         #pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) {
-            const int c = tid + i * NT, row = c / (kKT2 / 8), kc = c % (kKT2 / 8);
-            *reinterpret_cast<u32x4*>(&Xs[row * kLd2 + kc * 8]) = R.a[i];
-        }
-        #pragma unroll
-        for (int i = 0; i < B_CHUNKS; ++i) {
-            const int c = tid + i * NT, row = c / B_CPR, kc = c % B_CPR;
-            if constexpr (KIND == WK_I8) {
-                uint32_t h[8];
-                i8x4_to_h4(R.b[i].x, h[0], h[1]);
-                i8x4_to_h4(R.b[i].y, h[2], h[3]);
-                i8x4_to_h4(R.b[i].z, h[4], h[5]);
-                i8x4_to_h4(R.b[i].w, h[6], h[7]);
-                *reinterpret_cast<u32x4*>(&Ws[row * kLd2 + kc * 16]) = u32x4{h[0], h[1], h[2], h[3]};
-                *reinterpret_cast<u32x4*>(&Ws[row * kLd2 + kc * 16 + 8]) = u32x4{h[4], h[5], h[6], h[7]};
-            } else {
-                *reinterpret_cast<u32x4*>(&Ws[row * kLd2 + kc * 8]) = R.b[i];
+        for (int d = kStages - 2; d >= 1; --d) {
+            if (!done && stages >= d) {
+                MI_WAIT_VM(d * kLoads);
+                done = true;
             }
         }
-    };
-    auto multiply = [&](const uint16_t* Xs, const uint16_t* Ws) {
-        #pragma unroll
-        for (int kk = 0; kk < kKT2 / 16; ++kk) {
-            const int kcol = 16 * gk + 8 * kk;      // lane group gk supplies k = 16 gk + 8 kk .. +7
-            half8 w[TN], xf[TM];
-            #pragma unroll
-            for (int u = 0; u < TN; ++u)
-                w[u] = *reinterpret_cast<const half8*>(&Ws[(wn * 64 + u * 32 + li) * kLd2 + kcol]);
-            #pragma unroll
-            for (int t = 0; t < TM; ++t)
-                xf[t] = *reinterpret_cast<const half8*>(&Xs[(t * 32 + li) * kLd2 + kcol]);
-            #pragma unroll
-            for (int u = 0; u < TN; ++u)
-                #pragma unroll
-                for (int t = 0; t < TM; ++t)
-                    acc[u][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(w[u], xf[t], acc[u][t], 0, 0, 0);
-        }
+        if (!done) MI_WAIT_VM(0);
     };
 
-    const int nk = K / kKT2;
-    Regs R0, R1, R2;
-    load_tile(R0, 0);
-    load_tile(R1, (1 < nk ? 1 : nk - 1) * kKT2);
-    load_tile(R2, (2 < nk ? 2 : nk - 1) * kKT2);
-#define MI_GEMM2_STEP(R)                                                       \
-    {                                                                          \
-        uint16_t* Xs = lds + (i & 1) * kStage;                                 \
-        uint16_t* Ws = Xs + BM * kLd2;                                         \
-        store_tile(R, Xs, Ws);                                                 \
-        __syncthreads();                                                       \
-        load_tile(R, (i + 3 < nk ? i + 3 : nk - 1) * kKT2);                    \
-        multiply(Xs, Ws);                                                      \
-        if (++i >= nk) break;                                                  \
-    }
-    for (int i = 0;;) {
-        MI_GEMM2_STEP(R0)
-        MI_GEMM2_STEP(R1)
-        MI_GEMM2_STEP(R2)
-    }
-#undef MI_GEMM2_STEP
-
-    // D[i][j]: i = 8 (r / 4) + 4 (lane / 32) + r % 4 is a W row (an output column), j = lane % 32
-    // is a row of x (an output row): a lane holds 4 consecutive output columns per r / 4.
-    const bool vec_ok = (N % 4) == 0;
+    const int nk = K / 64;
+    Frags<TM> FA, FB;
     #pragma unroll
-    for (int u = 0; u < TN; ++u) {
+    for (int st = 0; st < kStages - 1; ++st)
+        if (st < nk) fill_stage(st, st);
+    wait_fills((nk < kStages - 1 ? nk : kStages - 1) - 1);          // stage 0 has landed
+    __builtin_amdgcn_s_barrier();
+    MI_SCHED_FENCE();
+    static_for<kReads>([&](auto jc) { read_one(FA, 0u, std::integral_constant<int, 0>{}, jc); });
+    MI_WAIT_LGKM(0);
+    MI_SCHED_FENCE();
+    static_for<8>([&](auto jc) { convert_one(FA, jc); });
+
+    // Stage i lives in slot i % kStages.  In the middle of stage i every wavefront waits for its
+    // own fills of stage i + 1 and meets the others at the barrier; behind it stage i + 1 is
+    // complete and stage i - 1 is no longer read, so its slot takes stage i + kStages - 1.
+    auto stage = [&](int i, int slot, auto fillc) {
+        const int next = slot + 1 == kStages ? 0 : slot + 1;
+        const int prev = slot == 0 ? kStages - 1 : slot - 1;
+        half_stage(FA, FB, static_cast<uint32_t>(slot) * kStage, std::integral_constant<int, 1>{},
+                   std::false_type{}, 0, 0);
+        MI_SCHED_FENCE();
+        const int last = i + kStages - 2 < nk - 1 ? i + kStages - 2 : nk - 1;   // newest stage requested so far
+        wait_fills(last - (i + 1));
+        __builtin_amdgcn_s_barrier();
+        MI_SCHED_FENCE();
+        // (after the last stage the fragments read here are not used)
+        half_stage(FB, FA, static_cast<uint32_t>(next) * kStage, std::integral_constant<int, 0>{},
+                   fillc, i + kStages - 1, prev);
+        MI_SCHED_FENCE();
+    };
+    int slot = 0, i = 0;
+    for (; i + kStages - 1 < nk; ++i) {
+        stage(i, slot, std::true_type{});
+        slot = slot + 1 == kStages ? 0 : slot + 1;
+    }
+    for (; i < nk; ++i) {
+        stage(i, slot, std::false_type{});
+        slot = slot + 1 == kStages ? 0 : slot + 1;
+    }
+
+    // --- epilogue ----------------------------------------------------------------------------------
+    // D[i][j]: i = 8 (r / 4) + 4 (lane / 32) + r % 4 is a row of W (an output column), j = lane % 32
+    // a row of x (an output row): a lane holds 4 consecutive output columns per r / 4.  The
+    // scaled fp16 values go through LDS (rows of 64 columns, padded to 144 bytes) so that the
+    // stores to out are 16 bytes per lane and 128 consecutive bytes per 8 lanes.
+    MI_WAIT_LGKM(0);
+    __builtin_amdgcn_s_barrier();                        // nobody reads operands from LDS any more
+    MI_SCHED_FENCE();
+    constexpr int kERow = 144;
+    uint8_t* ebase = lds + w * (BM * kERow);
+    #pragma unroll
+    for (int u = 0; u < 2; ++u) {
         #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
-            const int n = n0 + wn * 64 + u * 32 + 8 * rq + 4 * gk;      // first of 4 columns
-            float s4[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-            if constexpr (KIND == WK_I8) {
-                #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    s4[e] = __half2float(__ushort_as_half(scale[n + e < N ? n + e : N - 1]));
-            }
+            float s4[4];
+            s4[0] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].x & 0xFFFFu)));
+            s4[1] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].x >> 16)));
+            s4[2] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].y & 0xFFFFu)));
+            s4[3] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].y >> 16)));
             #pragma unroll
             for (int t = 0; t < TM; ++t) {
-                const int m = m0 + t * 32 + li;
-                if (m >= M) continue;
-                uint16_t h[4];
+                uint32_t h[4];
                 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float v = KIND == WK_I8 ? acc[u][t][4 * rq + e] * s4[e] : acc[u][t][4 * rq + e];
-                    h[e] = to_half_bits(v);
-                }
-                uint16_t* dst = out + static_cast<size_t>(m) * N + n;
-                if (vec_ok && n + 3 < N) {
-                    uint2 pk;
-                    pk.x = static_cast<uint32_t>(h[0]) | (static_cast<uint32_t>(h[1]) << 16);
-                    pk.y = static_cast<uint32_t>(h[2]) | (static_cast<uint32_t>(h[3]) << 16);
-                    *reinterpret_cast<uint2*>(dst) = pk;
-                } else {
-                    #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (n + e < N) dst[e] = h[e];
-                }
+                for (int e = 0; e < 4; ++e) h[e] = to_half_bits(acc[u][t][4 * rq + e] * s4[e]);
+                *reinterpret_cast<uint2*>(ebase + (32 * t + li) * kERow + (32 * u + 8 * rq + 4 * g) * 2) =
+                    uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
             }
+        }
+    }
+    // each wavefront reads back only what it wrote itself
+    const int ncol = n0 + 64 * w + 8 * (lane & 7);       // first of this lane's 8 output columns
+    const bool cols8 = (N % 8) == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    #pragma unroll
+    for (int j = 0; j < BM / 8; ++j) {
+        const int row = 8 * j + (lane >> 3);
+        const u32x4 v = *reinterpret_cast<const u32x4*>(ebase + row * kERow + (lane & 7) * 16);
+        const int m = m0 + row;
+        if (m >= M) continue;
+        uint16_t* dst = out + static_cast<size_t>(m) * N + ncol;
+        if (cols8 && ncol + 7 < N) {
+            *reinterpret_cast<u32x4*>(dst) = v;
+        } else {
+            #pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (ncol + e < N) dst[e] = static_cast<uint16_t>(v[e / 2] >> (16 * (e % 2)));
         }
     }
 }
 
-template <int KIND_UNUSED = 0>
-bool launch_128x128(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x, const void* W,
-                    const void* scale, void* out) {
-    const dim3 grid((N + 127) / 128, (M + 127) / 128, 1);
-    const auto* xp = static_cast<const uint16_t*>(x);
-    const auto* wp = static_cast<const uint8_t*>(W);
-    const auto* sp = static_cast<const uint16_t*>(scale);
-    auto* op = static_cast<uint16_t*>(out);
-    if (kind == WK_I8)
-        hipLaunchKernelGGL(gemm_kernel_128x128<WK_I8>, grid, dim3(128), 0, s, xp, wp, sp, op, M, N, K);
-    else
-        hipLaunchKernelGGL(gemm_kernel_128x128<WK_F16>, grid, dim3(128), 0, s, xp, wp, sp, op, M, N, K);
+template <int TM>
+bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out) {
+    constexpr size_t lds_bytes = static_cast<size_t>(stages_for(TM)) * (32 * TM * 128 + kWStage);
+    auto* kern = gemm_i8_wide<TM>;
+    static bool raised = false;
+    if (lds_bytes > 65536 && !raised) {
+        if (!MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes))) return false;
+        raised = true;
+    }
+    const dim3 grid((N + kBN - 1) / kBN, (M + 32 * TM - 1) / (32 * TM), 1);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, s, static_cast<const uint16_t*>(x),
+                       static_cast<const uint8_t*>(W), static_cast<const uint16_t*>(scale),
+                       static_cast<uint16_t*>(out), M, N, K);
     return MI_HIP_OK(hipGetLastError());
 }
+
+// Rows of x per block, in units of 32: the value whose estimated time (rounds of blocks over
+// the CUs x time of one block) is smallest.  A block's K-step of 16 costs the larger of its
+// MFMA time and its LDS time (fill at ~150 B/ns, fragment reads at ~530 B/ns).
+inline int pick_tm(int M, int N, int cus) {
+    int best = 1;
+    double best_t = 1e30;
+    for (int tm = 1; tm <= 5; ++tm) {
+        const long blocks = static_cast<long>((M + 32 * tm - 1) / (32 * tm)) * ((N + kBN - 1) / kBN);
+        const long rounds = (blocks + cus - 1) / cus;
+        const double mfma = 2.0 * tm * 15.6;
+        const double lds = (32.0 * tm * 32 + kBN * 16) / 150.0 + 4.0 * (tm + 1) * 1024 / 530.0;
+        const double t = rounds * ((mfma > lds ? mfma : lds) + 0.15 * (mfma < lds ? mfma : lds));
+        if (t < best_t) { best_t = t; best = tm; }
+    }
+    return best;
+}
+
+inline bool launch_any(int tm, hipStream_t s, int M, int N, int K, const void* x, const void* W,
+                       const void* scale, void* out) {
+    switch (tm) {
+        case 1: return launch<1>(s, M, N, K, x, W, scale, out);
+        case 2: return launch<2>(s, M, N, K, x, W, scale, out);
+        case 3: return launch<3>(s, M, N, K, x, W, scale, out);
+        case 4: return launch<4>(s, M, N, K, x, W, scale, out);
+        default: return launch<5>(s, M, N, K, x, W, scale, out);
+    }
+}
+
+}  // namespace wide
 
 template <int BM, int BN, int WM, int WN>
 bool launch_tile(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x, const void* W,
@@ -408,7 +599,14 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
     // 128 x 128 tiles once they fill every CU twice over (two blocks are resident per CU);
     // below that the 64 x 64 tile spreads the work over more CUs and wins (measured).
     const int mode = gemm_mode();
-    if (mode == 3) return launch_128x128<>(s, kind, M, N, K, x, W, scale, out);
+    if (kind == WK_I8 && (mode == 3 || (mode >= 11 && mode <= 15))) {
+        if (static_cast<double>(M) * K * 2 >= 4294967296.0 || static_cast<double>(N) * K >= 4294967296.0) {
+            MI_ERROR_FMT("gemm: operand larger than the 4 GB the wide kernel's 32-bit offsets cover");
+            return false;
+        }
+        const int tm = mode == 3 ? wide::pick_tm(M, N, device_info().cus) : mode - 10;
+        return wide::launch_any(tm, s, M, N, K, x, W, scale, out);
+    }
     if (mode != 2 && M > 64 && tiles(M, N, 128, 128) >= 2L * device_info().cus)
         return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);
     return launch_tile<64, 64, 32, 32>(s, kind, M, N, K, x, W, scale, out);

@@ -122,8 +122,9 @@ int   mi_graph_destroy(void* graph);
 /* Selects how M > 1 is computed for a quantised W: 0 (default) = MFMA GEMM with fused
  * dequant for M >= 16 and batched GEMV below; 1 = always the batched GEMV, whose rows
  * are bit-identical to M = 1 calls (the reference's prefill loop, LF/src/model.cpp:243-250);
- * 2 and 3 = as 0 with the tile choice pinned to the 64 x 64 resp. 128 x 128 kernel (tests
- * and tuning: results stay within the same tolerance, only the speed differs). */
+ * 2, 3 and 11..15 = as 0 with the kernel choice pinned (tests and tuning: results stay within
+ * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel, 3 = the wide int8
+ * kernel, 10 + t = the wide int8 kernel with 32 t rows of x per block. */
 void mi_set_gemm_mode(int mode);
 
 /* Selects the M = 1 arithmetic.  0 = every GEMV evaluates the reference kernels' sum in the

@@ -35,7 +35,8 @@ def _ulp_apart(a_u16, b_u16):
 
 def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0):
     """tile is the mi_set_gemm_mode value: 0 = the library's own choice, 1 = rows of GEMV,
-    2 / 3 = the 64 x 64 / 128 x 128 MFMA kernel."""
+    2 = the 64 x 64 MFMA kernel, 3 = the wide int8 kernel with its own choice of rows of x per
+    block, 11..15 = the wide kernel with 32, 64, .. 160 rows of x per block."""
     xb, wb = mil.Buffer.from_host(X), mil.Buffer.from_host(W_host)
     sb = mil.Buffer.from_host(scale_host) if scale_host is not None else None
     if kind == "i8":
@@ -55,7 +56,7 @@ def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0):
     return full[pad:-pad].reshape(M, N)
 
 
-@pytest.mark.parametrize("tile", [2, 3])
+@pytest.mark.parametrize("tile", [2, 3, 11, 12, 13, 14, 15])
 @pytest.mark.parametrize("M", [16, 64, 100, 512])
 @pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (200, 128), (130, 576), (131, 64)])
 def test_int8_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
@@ -81,7 +82,7 @@ def test_fp16_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
     assert _ulp_apart(got, want).max() <= 1
 
 
-@pytest.mark.parametrize("tile", [2, 3])
+@pytest.mark.parametrize("tile", [2, 3, 11, 13, 15])
 def test_gemm_exact_on_integer_data(queue, tile):
     # small integers: every partial sum is exact in fp32, so any summation order gives the same bits
     rng = np.random.default_rng(3)
@@ -95,7 +96,7 @@ def test_gemm_exact_on_integer_data(queue, tile):
     assert np.array_equal(got, O.gemm_i8(X, q, s.view(np.uint16)))
 
 
-@pytest.mark.parametrize("tile", [2, 3])
+@pytest.mark.parametrize("tile", [2, 3, 12, 14, 15])
 def test_gemm_unit_rows_pick_weight_columns(queue, tile):
     # x rows are unit vectors: out[i, :] must be the dequantised column k_i of W (index check)
     M, N, K = 64, 320, 896
@@ -107,6 +108,32 @@ def test_gemm_unit_rows_pick_weight_columns(queue, tile):
     got = _gemm(queue, M, N, K, X, q, s, "i8", tile).view(np.float16)
     want = (q[:, ks].T.astype(np.float32) * s.astype(np.float32)[None, :]).astype(np.float16)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("tile", [2, 11, 12, 13, 14, 15])
+def test_gemm_repeats_identically(queue, tile):
+    """The same launch 25 times: every result identical to the first and within tolerance of the
+    oracle (a race between the LDS fills, the fragment reads and the barriers would show here)."""
+    M, N, K = 100, 1000, 1024
+    print(f"repeat tile mode {tile}", flush=True)
+    W, X = synth_w(940, N, K), synth_x(941, M, K)
+    q, s = mil.quantize_int8(W)
+    want = O.gemm_i8(X, q, s.view(np.uint16))
+    xb, wb, sb = mil.Buffer.from_host(X), mil.Buffer.from_host(q), mil.Buffer.from_host(s)
+    assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+    outs = [mil.Buffer(M * N * 2) for _ in range(25)]
+    mil.lib().mi_set_gemm_mode(tile)
+    try:
+        for ob in outs:
+            assert mil.pytorch_linear(queue, M, N, K, xb, wb, ob)
+        queue.finish()
+    finally:
+        mil.lib().mi_set_gemm_mode(0)
+    first = outs[0].read(np.uint16, (M, N))
+    assert_tolerance(first.view(np.float16), want.view(np.float16))
+    for i, ob in enumerate(outs[1:]):
+        assert np.array_equal(ob.read(np.uint16, (M, N)), first), f"launch {i + 1} differs from launch 0"
+    mil.nnopt_unregister_weight(wb)
 
 
 def test_prefill_size_rows_sampled(queue):
