@@ -230,6 +230,16 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
 
+typedef float float2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+// two fp32 values, already rounded to fp32, to a pair of fp16 (round to nearest even): one
+// v_cvt_pk_f16_f32
+__device__ __forceinline__ uint32_t pack_half2(float a, float b) {
+    float2v v = {a, b};
+    asm volatile("" : "+v"(v));    // keep the fp32 rounding of the products: no fused multiply-convert
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, half2v));
+}
+
 template <int TM>
 struct Frags {
     u32x4 w[2];          // 16 int8 of two 32-row fragments of W, as read from LDS
@@ -469,11 +479,9 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
             s4[3] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].y >> 16)));
             #pragma unroll
             for (int t = 0; t < TM; ++t) {
-                uint32_t h[4];
-                #pragma unroll
-                for (int e = 0; e < 4; ++e) h[e] = to_half_bits(acc[u][t][4 * rq + e] * s4[e]);
-                *reinterpret_cast<uint2*>(ebase + (32 * t + li) * kERow + (32 * u + 8 * rq + 4 * g) * 2) =
-                    uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+                const uint32_t lo = pack_half2(acc[u][t][4 * rq] * s4[0], acc[u][t][4 * rq + 1] * s4[1]);
+                const uint32_t hi = pack_half2(acc[u][t][4 * rq + 2] * s4[2], acc[u][t][4 * rq + 3] * s4[3]);
+                *reinterpret_cast<uint2*>(ebase + (32 * t + li) * kERow + (32 * u + 8 * rq + 4 * g) * 2) = uint2{lo, hi};
             }
         }
     }
@@ -514,20 +522,26 @@ bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, co
     return MI_HIP_OK(hipGetLastError());
 }
 
-// Rows of x per block, in units of 32: the value whose estimated time (rounds of blocks over
-// the CUs x time of one block) is smallest.  A block's K-step of 16 costs the larger of its
-// MFMA time and its LDS time (fill at ~150 B/ns, fragment reads at ~530 B/ns).
-inline int pick_tm(int M, int N, int cus) {
+// Estimated time (us) of the wide kernel with 32 * tm rows of x per block.  Fitted to
+// measurements on MI355X: a block takes about 2.6 + 0.5 tm us of prologue and epilogue plus, per
+// K-stage of 64, 0.27 + 0.10 tm us; a fully occupied chip runs the same cycles about 1.56 times
+// slower (clock under load, shared L2 and fabric) than a nearly empty one.
+inline double estimate_us(int tm, int M, int N, int K, int cus) {
+    const long blocks = static_cast<long>((M + 32 * tm - 1) / (32 * tm)) * ((N + kBN - 1) / kBN);
+    const double block_us = 2.6 + 0.5 * tm + (K / 64) * (0.27 + 0.10 * tm);
+    const long full = blocks / cus, rem = blocks % cus;
+    return full * 1.56 * block_us + (rem ? (1.0 + 0.56 * rem / cus) * block_us : 0.0);
+}
+
+// Rows of x per block, in units of 32: the value with the smallest estimated time.
+inline int pick_tm(int M, int N, int K, int cus, double* best_us) {
     int best = 1;
     double best_t = 1e30;
     for (int tm = 1; tm <= 5; ++tm) {
-        const long blocks = static_cast<long>((M + 32 * tm - 1) / (32 * tm)) * ((N + kBN - 1) / kBN);
-        const long rounds = (blocks + cus - 1) / cus;
-        const double mfma = 2.0 * tm * 15.6;
-        const double lds = (32.0 * tm * 32 + kBN * 16) / 150.0 + 4.0 * (tm + 1) * 1024 / 530.0;
-        const double t = rounds * ((mfma > lds ? mfma : lds) + 0.15 * (mfma < lds ? mfma : lds));
+        const double t = estimate_us(tm, M, N, K, cus);
         if (t < best_t) { best_t = t; best = tm; }
     }
+    if (best_us) *best_us = best_t;
     return best;
 }
 
@@ -596,18 +610,31 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
         MI_ERROR_FMT("gemm: x and W must be 16-byte aligned, int8 needs a scale");
         return false;
     }
+    const int mode = gemm_mode();
+    const int cus = device_info().cus;
+    // int8: the wide kernel where its estimated time beats that of the 64 x 64 tiles, which are
+    // bound either by one tile's serial K loop (about 0.4 us per K-tile, up to 1.3 times that as
+    // the chip fills) or by throughput (1.2 to 1.55 ns per tile and K-tile); fitted to measurements
+    const bool wide_fits = kind == WK_I8 && static_cast<double>(M) * K * 2 < 4294967296.0 &&
+                           static_cast<double>(N) * K < 4294967296.0;   // 32-bit byte offsets
+    if (wide_fits && (mode == 0 || mode == 3 || (mode >= 11 && mode <= 15))) {
+        double wide_us = 0.0;
+        int tm = wide::pick_tm(M, N, K, cus, &wide_us);
+        const int nk = K / kKT;
+        const long t64 = tiles(M, N, 64, 64);
+        const double serial = (0.9 + nk * 0.4) * (1.0 + 0.3 * (t64 < 128 ? t64 / 128.0 : 1.0));
+        const double bulk = 3.3 + t64 * nk * (nk > 32 ? 0.00155 : 0.0012);
+        const double tiled_us = serial > bulk ? serial : bulk;
+        if (mode >= 11) tm = mode - 10;
+        if (mode != 0 || wide_us < tiled_us) return wide::launch_any(tm, s, M, N, K, x, W, scale, out);
+    } else if (mode == 3 || mode >= 11) {
+        MI_ERROR_FMT("gemm: mode %d asks for the wide int8 kernel, which does not take kind=%d M=%d N=%d K=%d",
+                     mode, static_cast<int>(kind), M, N, K);
+        return false;
+    }
     // 128 x 128 tiles once they fill every CU twice over (two blocks are resident per CU);
     // below that the 64 x 64 tile spreads the work over more CUs and wins (measured).
-    const int mode = gemm_mode();
-    if (kind == WK_I8 && (mode == 3 || (mode >= 11 && mode <= 15))) {
-        if (static_cast<double>(M) * K * 2 >= 4294967296.0 || static_cast<double>(N) * K >= 4294967296.0) {
-            MI_ERROR_FMT("gemm: operand larger than the 4 GB the wide kernel's 32-bit offsets cover");
-            return false;
-        }
-        const int tm = mode == 3 ? wide::pick_tm(M, N, device_info().cus) : mode - 10;
-        return wide::launch_any(tm, s, M, N, K, x, W, scale, out);
-    }
-    if (mode != 2 && M > 64 && tiles(M, N, 128, 128) >= 2L * device_info().cus)
+    if (mode != 2 && M > 64 && tiles(M, N, 128, 128) >= 2L * cus)
         return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);
     return launch_tile<64, 64, 32, 32>(s, kind, M, N, K, x, W, scale, out);
 }

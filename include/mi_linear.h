@@ -124,7 +124,8 @@ int   mi_graph_destroy(void* graph);
  * are bit-identical to M = 1 calls (the reference's prefill loop, LF/src/model.cpp:243-250);
  * 2, 3 and 11..15 = as 0 with the kernel choice pinned (tests and tuning: results stay within
  * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel, 3 = the wide int8
- * kernel, 10 + t = the wide int8 kernel with 32 t rows of x per block. */
+ * kernel, 10 + t (t = 1..5) = the wide int8 kernel with 32 t rows of x per block; 3 and 10 + t
+ * fail for weights that are not int8. */
 void mi_set_gemm_mode(int mode);
 
 /* Selects the M = 1 arithmetic.  0 = every GEMV evaluates the reference kernels' sum in the

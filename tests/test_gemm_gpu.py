@@ -36,7 +36,7 @@ def _ulp_apart(a_u16, b_u16):
 def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0):
     """tile is the mi_set_gemm_mode value: 0 = the library's own choice, 1 = rows of GEMV,
     2 = the 64 x 64 MFMA kernel, 3 = the wide int8 kernel with its own choice of rows of x per
-    block, 11..15 = the wide kernel with 32, 64, .. 160 rows of x per block."""
+    block, 11..15 = the wide kernel with 32, 64, .. 160 rows of x per block (int8 only)."""
     xb, wb = mil.Buffer.from_host(X), mil.Buffer.from_host(W_host)
     sb = mil.Buffer.from_host(scale_host) if scale_host is not None else None
     if kind == "i8":
@@ -56,7 +56,7 @@ def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0):
     return full[pad:-pad].reshape(M, N)
 
 
-@pytest.mark.parametrize("tile", [2, 3, 11, 12, 13, 14, 15])
+@pytest.mark.parametrize("tile", [0, 2, 3, 11, 12, 13, 14, 15])
 @pytest.mark.parametrize("M", [16, 64, 100, 512])
 @pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (200, 128), (130, 576), (131, 64)])
 def test_int8_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
@@ -71,8 +71,9 @@ def test_int8_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
     assert np.mean(got == want) > 0.99
 
 
-@pytest.mark.parametrize("tile", [2, 3])
-@pytest.mark.parametrize("M,N,K", [(64, 4864, 896), (256, 896, 4864), (33, 200, 128), (130, 131, 64)])
+@pytest.mark.parametrize("tile", [0, 2])
+@pytest.mark.parametrize("M,N,K", [(64, 4864, 896), (256, 896, 4864), (33, 200, 128), (130, 131, 64),
+                                   (2048, 4864, 128)])   # the last one takes the 128 x 128 tiles in mode 0
 def test_fp16_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
     print(f"fp16 gemm M={M} N={N} K={K} tile mode {tile}", flush=True)
     W, X = synth_w(900 + N, N, K), synth_x(901 + M, M, K)
