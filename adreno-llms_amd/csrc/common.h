@@ -58,7 +58,9 @@ bool launch_unpack_q4(hipStream_t s, const void* p, int N, int K, void* w8);
 
 // gemm.hip: out[M,N] = x[M,K] W^T on MFMA with the dequant fused into the tile load.
 bool gemm_supported(WeightKind kind, int M, int N, int K);
+// workspace: device memory that belongs to stream s (or null): the int8 kernel may cut K into
+// slices and park fp32 partial sums there; calls on one stream are ordered, so they can share it.
 bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x,
-                 const void* W, const void* scale, void* out);
+                 const void* W, const void* scale, void* out, void* workspace, size_t workspace_bytes);
 
 }  // namespace mi

@@ -251,7 +251,8 @@ template <int TM>
 __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__ X,
                                                    const uint8_t* __restrict__ W,
                                                    const uint16_t* __restrict__ scale,
-                                                   uint16_t* __restrict__ out, int M, int N, int K) {
+                                                   uint16_t* __restrict__ out, int M, int N, int K,
+                                                   float* __restrict__ partial, int splits) {
     constexpr int BM = 32 * TM;
     constexpr int kXStage = BM * 128;                    // bytes of x (fp16) per stage
     constexpr int kStage = kXStage + kWStage;
@@ -264,7 +265,29 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane >> 5, li = lane & 31;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * kBN;
+    // Block -> tile.  Blocks go to the 8 XCDs round-robin and every XCD has its own L2, so XCD x
+    // takes the x-th contiguous eighth of the tile list, and the list runs through bands of 4
+    // tiles along N, down M inside a band: the tiles that are in flight on one XCD at the same
+    // time then share rows of x and of W and fetch them into that L2 once.
+    // With splits > 1 the list holds every tile once per slice of K (slice-major); a block then
+    // sums its slice only and leaves fp32 partial sums for reduce_partials.
+    int tile_m, tile_n, split;
+    {
+        const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + kBN - 1) / kBN, tiles = tiles_m * tiles_n;
+        const int total = tiles * splits;
+        const int per_xcd = (total + 7) / 8;
+        int l = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+        if (blockIdx.x >= 8 * per_xcd || l >= total) return;          // whole block, before any barrier
+        split = l / tiles;
+        l -= split * tiles;
+        constexpr int kBand = 4;
+        const int band = l / (kBand * tiles_m);
+        const int width = tiles_n - band * kBand < kBand ? tiles_n - band * kBand : kBand;
+        const int in_band = l - band * kBand * tiles_m;
+        tile_m = in_band / width;
+        tile_n = band * kBand + in_band % width;
+    }
+    const int m0 = tile_m * BM, n0 = tile_n * kBN;
     const uint32_t lbase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_u8*)lds));
 
     // per-row scales of this lane's output columns, requested before anything else so that they
@@ -305,7 +328,7 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
         const int n = n0 + r < N ? n0 + r : N - 1;
         wsrc[jj] = static_cast<uint32_t>(n) * K + c * 16u;
     }
-    const uint8_t* Xb = reinterpret_cast<const uint8_t*>(X);
+    const uint8_t* Xb = reinterpret_cast<const uint8_t*>(X);     // both advanced to the block's first K-stage below
     // load j (0 .. kLoads - 1) of this wavefront for K-stage stage_k into LDS slot `slot`
     auto fill_one = [&](int stage_k, int slot, auto jc) {
         constexpr int j = decltype(jc)::value;
@@ -417,7 +440,11 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
         if (!done) MI_WAIT_VM(0);
     };
 
-    const int nk = K / 64;
+    // this block's K-stages: [k_first, k_first + nk) of the K / 64 stages
+    const int k_first = static_cast<int>(static_cast<long>(K / 64) * split / splits);
+    const int nk = static_cast<int>(static_cast<long>(K / 64) * (split + 1) / splits) - k_first;
+    Xb += static_cast<size_t>(k_first) * 128;
+    W += static_cast<size_t>(k_first) * 64;
     Frags<TM> FA, FB;
     #pragma unroll
     for (int st = 0; st < kStages - 1; ++st)
@@ -463,6 +490,33 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
     // a row of x (an output row): a lane holds 4 consecutive output columns per r / 4.  The
     // scaled fp16 values go through LDS (rows of 64 columns, padded to 144 bytes) so that the
     // stores to out are 16 bytes per lane and 128 consecutive bytes per 8 lanes.
+    if (partial) {
+        // slice of K: the raw fp32 sums, 16 bytes per lane, into partial[split][M][N]
+        float* pout = partial + static_cast<size_t>(split) * M * N;
+        const bool vec4 = (N % 4) == 0;
+        #pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            #pragma unroll
+            for (int rq = 0; rq < 4; ++rq) {
+                const int nq = n0 + 64 * w + 32 * u + 8 * rq + 4 * g;
+                #pragma unroll
+                for (int t = 0; t < TM; ++t) {
+                    const int m = m0 + 32 * t + li;
+                    if (m >= M) continue;
+                    float* dst = pout + static_cast<size_t>(m) * N + nq;
+                    if (vec4 && nq + 3 < N) {
+                        *reinterpret_cast<float4*>(dst) = float4{acc[u][t][4 * rq], acc[u][t][4 * rq + 1],
+                                                                 acc[u][t][4 * rq + 2], acc[u][t][4 * rq + 3]};
+                    } else {
+                        #pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (nq + e < N) dst[e] = acc[u][t][4 * rq + e];
+                    }
+                }
+            }
+        }
+        return;
+    }
     MI_WAIT_LGKM(0);
     __builtin_amdgcn_s_barrier();                        // nobody reads operands from LDS any more
     MI_SCHED_FENCE();
@@ -505,8 +559,36 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
     }
 }
 
+// out[m][n] = fp16((sum over slices of partial[slice][m][n]) * scale[n]); slices are added in
+// index order, so the result does not depend on how the blocks were scheduled.
+__global__ __launch_bounds__(256) void reduce_partials(const float* __restrict__ partial, int splits,
+                                                       const uint16_t* __restrict__ scale,
+                                                       uint16_t* __restrict__ out, long MN, int N) {
+    const long i4 = (static_cast<long>(blockIdx.x) * 256 + threadIdx.x) * 4;
+    if (i4 >= MN) return;
+    const bool vec = (N % 4) == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0;
+    if (vec) {
+        float4 a = *reinterpret_cast<const float4*>(partial + i4);
+        for (int z = 1; z < splits; ++z) {
+            const float4 b = *reinterpret_cast<const float4*>(partial + z * MN + i4);
+            a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+        }
+        const int n = static_cast<int>(i4 % N);
+        const float s0 = __half2float(__ushort_as_half(scale[n])), s1 = __half2float(__ushort_as_half(scale[n + 1]));
+        const float s2 = __half2float(__ushort_as_half(scale[n + 2])), s3 = __half2float(__ushort_as_half(scale[n + 3]));
+        *reinterpret_cast<uint2*>(out + i4) = uint2{pack_half2(a.x * s0, a.y * s1), pack_half2(a.z * s2, a.w * s3)};
+    } else {
+        for (int e = 0; e < 4 && i4 + e < MN; ++e) {
+            float a = partial[i4 + e];
+            for (int z = 1; z < splits; ++z) a += partial[z * MN + i4 + e];
+            out[i4 + e] = to_half_bits(a * __half2float(__ushort_as_half(scale[(i4 + e) % N])));
+        }
+    }
+}
+
 template <int TM>
-bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out) {
+bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out,
+            float* partial, int splits) {
     constexpr size_t lds_bytes = static_cast<size_t>(stages_for(TM)) * (32 * TM * 128 + kWStage);
     auto* kern = gemm_i8_wide<TM>;
     static bool raised = false;
@@ -515,44 +597,61 @@ bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, co
                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes))) return false;
         raised = true;
     }
-    const dim3 grid((N + kBN - 1) / kBN, (M + 32 * TM - 1) / (32 * TM), 1);
+    const long total = static_cast<long>((N + kBN - 1) / kBN) * ((M + 32 * TM - 1) / (32 * TM)) * splits;
+    const dim3 grid(static_cast<unsigned>(8 * ((total + 7) / 8)), 1, 1);      // see the block -> tile map in the kernel
     hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, s, static_cast<const uint16_t*>(x),
                        static_cast<const uint8_t*>(W), static_cast<const uint16_t*>(scale),
-                       static_cast<uint16_t*>(out), M, N, K);
-    return MI_HIP_OK(hipGetLastError());
+                       static_cast<uint16_t*>(out), M, N, K, splits > 1 ? partial : nullptr, splits);
+    if (!MI_HIP_OK(hipGetLastError())) return false;
+    if (splits > 1) {
+        const long MN = static_cast<long>(M) * N;
+        hipLaunchKernelGGL(reduce_partials, dim3(static_cast<unsigned>((MN / 4 + 256) / 256)), dim3(256), 0, s,
+                           partial, splits, static_cast<const uint16_t*>(scale), static_cast<uint16_t*>(out), MN, N);
+        if (!MI_HIP_OK(hipGetLastError())) return false;
+    }
+    return true;
 }
 
-// Estimated time (us) of the wide kernel with 32 * tm rows of x per block.  Fitted to
-// measurements on MI355X: a block takes about 2.6 + 0.5 tm us of prologue and epilogue plus, per
-// K-stage of 64, 0.27 + 0.10 tm us; a fully occupied chip runs the same cycles about 1.56 times
-// slower (clock under load, shared L2 and fabric) than a nearly empty one.
-inline double estimate_us(int tm, int M, int N, int K, int cus) {
-    const long blocks = static_cast<long>((M + 32 * tm - 1) / (32 * tm)) * ((N + kBN - 1) / kBN);
-    const double block_us = 2.6 + 0.5 * tm + (K / 64) * (0.27 + 0.10 * tm);
+// Estimated time (us) of the wide kernel with 32 * tm rows of x per block and K cut into
+// `splits` slices.  Fitted to measurements on MI355X: a block takes about 2.6 + 0.5 tm us of
+// prologue and epilogue plus, per K-stage of 64, 0.27 + 0.10 tm us; a fully occupied chip runs
+// the same cycles about 1.56 times slower (clock under load, shared L2 and fabric) than a nearly
+// empty one.  Slices cost a second launch and the partial sums' trip through memory.
+inline double estimate_us(int tm, int splits, int M, int N, int K, int cus) {
+    const long blocks = static_cast<long>((M + 32 * tm - 1) / (32 * tm)) * ((N + kBN - 1) / kBN) * splits;
+    const int stages = (K / 64 + splits - 1) / splits;
+    const double block_us = 2.6 + 0.5 * tm + stages * (0.27 + 0.10 * tm);
     const long full = blocks / cus, rem = blocks % cus;
-    return full * 1.56 * block_us + (rem ? (1.0 + 0.56 * rem / cus) * block_us : 0.0);
+    double t = full * 1.56 * block_us + (rem ? (1.0 + 0.56 * rem / cus) * block_us : 0.0);
+    if (splits > 1) t += 2.5 + 2.0 * splits * M * static_cast<double>(N) * 4 / 4.0e6;   // ~4 TB/s there and back
+    return t;
 }
 
-// Rows of x per block, in units of 32: the value with the smallest estimated time.
-inline int pick_tm(int M, int N, int K, int cus, double* best_us) {
-    int best = 1;
+// Rows of x per block (in units of 32) and slices of K with the smallest estimated time; slices
+// only as far as their fp32 partial sums fit the workspace.
+inline void pick_shape(int M, int N, int K, int cus, size_t workspace_bytes, int* tm_out, int* splits_out,
+                       double* best_us) {
+    static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24};
     double best_t = 1e30;
     for (int tm = 1; tm <= 5; ++tm) {
-        const double t = estimate_us(tm, M, N, K, cus);
-        if (t < best_t) { best_t = t; best = tm; }
+        for (int sp : kSplits) {
+            if (sp > 1 && (K / 64 < 2 * sp || static_cast<double>(sp) * M * N * 4 > static_cast<double>(workspace_bytes)))
+                continue;
+            const double t = estimate_us(tm, sp, M, N, K, cus);
+            if (t < best_t) { best_t = t; *tm_out = tm; *splits_out = sp; }
+        }
     }
     if (best_us) *best_us = best_t;
-    return best;
 }
 
 inline bool launch_any(int tm, hipStream_t s, int M, int N, int K, const void* x, const void* W,
-                       const void* scale, void* out) {
+                       const void* scale, void* out, float* partial, int splits) {
     switch (tm) {
-        case 1: return launch<1>(s, M, N, K, x, W, scale, out);
-        case 2: return launch<2>(s, M, N, K, x, W, scale, out);
-        case 3: return launch<3>(s, M, N, K, x, W, scale, out);
-        case 4: return launch<4>(s, M, N, K, x, W, scale, out);
-        default: return launch<5>(s, M, N, K, x, W, scale, out);
+        case 1: return launch<1>(s, M, N, K, x, W, scale, out, partial, splits);
+        case 2: return launch<2>(s, M, N, K, x, W, scale, out, partial, splits);
+        case 3: return launch<3>(s, M, N, K, x, W, scale, out, partial, splits);
+        case 4: return launch<4>(s, M, N, K, x, W, scale, out, partial, splits);
+        default: return launch<5>(s, M, N, K, x, W, scale, out, partial, splits);
     }
 }
 
@@ -600,7 +699,7 @@ bool gemm_supported(WeightKind kind, int M, int N, int K) {
 }
 
 bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x, const void* W,
-                 const void* scale, void* out) {
+                 const void* scale, void* out, void* workspace, size_t workspace_bytes) {
     if (!gemm_supported(kind, M, N, K)) {
         MI_ERROR_FMT("gemm: unsupported kind=%d M=%d N=%d K=%d", static_cast<int>(kind), M, N, K);
         return false;
@@ -619,14 +718,17 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
                            static_cast<double>(N) * K < 4294967296.0;   // 32-bit byte offsets
     if (wide_fits && (mode == 0 || mode == 3 || (mode >= 11 && mode <= 15))) {
         double wide_us = 0.0;
-        int tm = wide::pick_tm(M, N, K, cus, &wide_us);
+        int tm = 1, splits = 1;
+        // modes 3 and 11..15 pin the plain kernel; slices of K are the library's own choice (mode 0)
+        wide::pick_shape(M, N, K, cus, mode == 0 && workspace ? workspace_bytes : 0, &tm, &splits, &wide_us);
         const int nk = K / kKT;
         const long t64 = tiles(M, N, 64, 64);
         const double serial = (0.9 + nk * 0.4) * (1.0 + 0.3 * (t64 < 128 ? t64 / 128.0 : 1.0));
         const double bulk = 3.3 + t64 * nk * (nk > 32 ? 0.00155 : 0.0012);
         const double tiled_us = serial > bulk ? serial : bulk;
         if (mode >= 11) tm = mode - 10;
-        if (mode != 0 || wide_us < tiled_us) return wide::launch_any(tm, s, M, N, K, x, W, scale, out);
+        if (mode != 0 || wide_us < tiled_us)
+            return wide::launch_any(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), splits);
     } else if (mode == 3 || mode >= 11) {
         MI_ERROR_FMT("gemm: mode %d asks for the wide int8 kernel, which does not take kind=%d M=%d N=%d K=%d",
                      mode, static_cast<int>(kind), M, N, K);

@@ -26,6 +26,29 @@ struct Entry {
 std::unordered_map<const void*, Entry> g_registry;
 std::mutex g_registry_mu;
 
+// One GEMM workspace per stream made by mi_stream_create, and one for the null stream made by
+// mi_init: allocated there, never inside a compute call.  Work on one stream is ordered, so the
+// calls of a stream can share its workspace; a stream from elsewhere has none and its GEMMs
+// simply do not slice K.
+constexpr size_t kWorkspaceBytes = 16u << 20;
+std::unordered_map<hipStream_t, void*> g_workspace;
+
+void* workspace_of(hipStream_t s) {
+    std::lock_guard<std::mutex> lk(g_registry_mu);
+    auto it = g_workspace.find(s);
+    return it == g_workspace.end() ? nullptr : it->second;
+}
+
+void add_workspace(hipStream_t s) {
+    void* p = nullptr;
+    if (hipMalloc(&p, kWorkspaceBytes) != hipSuccess) {
+        (void)hipGetLastError();      // no workspace: that stream's GEMMs run unsliced
+        return;
+    }
+    std::lock_guard<std::mutex> lk(g_registry_mu);
+    g_workspace[s] = p;
+}
+
 bool ensure_init() {
     if (g_inited) return true;
     return mi_init(0) == 1;
@@ -85,6 +108,7 @@ int mi_init(int device) {
     g_dev.device = device;
     g_dev.cus = prop.multiProcessorCount;
     std::snprintf(g_dev.arch, sizeof(g_dev.arch), "%s", prop.gcnArchName);
+    if (!g_inited && !workspace_of(nullptr)) add_workspace(nullptr);      // the null stream's GEMM workspace
     g_inited = true;
     return 1;
 }
@@ -127,10 +151,25 @@ void* mi_stream_create(void) {
     if (!ensure_init()) return nullptr;
     hipStream_t s = nullptr;
     if (!MI_HIP_OK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking))) return nullptr;
+    add_workspace(s);
     return s;
 }
 
-int mi_stream_destroy(void* s) { return s ? (MI_HIP_OK(hipStreamDestroy(as_stream(s))) ? 1 : 0) : 1; }
+int mi_stream_destroy(void* s) {
+    if (!s) return 1;
+    const int ok = MI_HIP_OK(hipStreamDestroy(as_stream(s))) ? 1 : 0;    // waits for the stream's work
+    void* ws = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(g_registry_mu);
+        auto it = g_workspace.find(as_stream(s));
+        if (it != g_workspace.end()) {
+            ws = it->second;
+            g_workspace.erase(it);
+        }
+    }
+    if (ws) (void)hipFree(ws);
+    return ok;
+}
 int mi_stream_sync(void* s) { return MI_HIP_OK(hipStreamSynchronize(as_stream(s))) ? 1 : 0; }
 
 void* mi_event_create(void) {
@@ -197,7 +236,8 @@ int mi_linear(void* stream, int M, int N, int K, const void* x, const void* W, v
     // M > 1: a real contraction goes to the MFMA GEMM; small batches, and every batch in
     // mode 1, run the GEMV once per row of x, as the reference's quantised prefill does.
     if (M >= 16 && g_gemm_mode != 1 && gemm_supported(e.kind, M, N, K))
-        return launch_gemm(as_stream(stream), e.kind, M, N, K, x, W, e.scale, out) ? 1 : 0;
+        return launch_gemm(as_stream(stream), e.kind, M, N, K, x, W, e.scale, out, workspace_of(as_stream(stream)),
+                           kWorkspaceBytes) ? 1 : 0;
     GemvCall c;
     c.x = x; c.W = W; c.scale = e.scale; c.y = out;
     c.M = M; c.N = N; c.K = K; c.kind = e.kind; c.epi = EPI_STORE;
