@@ -196,10 +196,15 @@ def main():
                     mil.linear_batch(queue, arr)
                 g.launch()
                 ms = min(ms, time_region(mil, queue, g.launch, 5) / len(arr))
+            # warm: the same weights every launch (they stay in the last-level cache)
+            warm = mil.make_calls([(1, N, K, xb, pool[0][0], yb)] * 32)
+            mil.linear_batch(queue, warm)
+            ms_warm = time_region(mil, queue, lambda: mil.linear_batch(queue, warm), 5) / 32
             for wb, _ in pool:
                 mil.nnopt_unregister_weight(wb)
             return {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
-                    "frac_hbm": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "bytes": nbytes}
+                    "frac_hbm": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "bytes": nbytes,
+                    "us_warm": round(ms_warm * 1e3, 2)}
 
         detail["c1_fp16_gemv_1536x576"] = cold_gemv("f16", 1536, 576, 340)
         detail["c2_int8_gemv_4864x896"] = cold_gemv("i8", INTER, H, 140)
@@ -249,6 +254,35 @@ def main():
             sample_bytes += VOCAB * H + 2 * VOCAB
             reps += 1
         dt = time.time() - t0
+        # per config, beside the GPU figures in `detail`: the same call on the host, all threads
+        # and one thread (bounded: each timed for about 0.3 s)
+        if not args.no_detail:
+            def cpu_us(fn):
+                fn()
+                t, n = time.time(), 0
+                while time.time() - t < 0.3 or n < 1:
+                    fn()
+                    n += 1
+                return round((time.time() - t) / n * 1e6, 1)
+
+            w1 = mil.synth_normal_f16(31, 0.02, (1536, 576))
+            x1 = mil.synth_normal_f16(32, 1.0, (576,))
+            gq, gs = host_layer0["gate"]
+            dq, ds = host_layer0["down"]
+            lp, lsc = mil.quantize_q4(mil.synth_normal_f16(7, 0.02, (VOCAB, H)))
+            X16 = mil.synth_normal_f16(78, 1.0, (16, H))
+            cases = {
+                "c1_fp16_gemv_1536x576": lambda t: O.gemv_f16(x1, w1, t),
+                "c2_int8_gemv_4864x896": lambda t: O.gemv_i8(xh, gq, gs.view(np.uint16), t),
+                "c2_int8_gemv_896x4864": lambda t: O.gemv_i8(xi, dq, ds.view(np.uint16), t),
+                "c3_int8_gemv_151936x896": lambda t: O.gemv_i8(xh, lm_host[0], lm_host[1].view(np.uint16), t),
+                "c3_q4_gemv_151936x896": lambda t: O.gemv_q4(xh, lp, lsc.view(np.uint16), t),
+                "c5_int8_gemm_M16_N4864_K896": lambda t: O.gemm_i8(X16, gq, gs.view(np.uint16), t),
+            }
+            detail["cpu_port"] = {"cores": threads}
+            for name, fn in cases.items():
+                detail["cpu_port"][name] = {"us_all_cores": cpu_us(lambda: fn(threads)),
+                                            "us_one_core": cpu_us(lambda: fn(1))}
         cpu = {"value": round(sample_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
                "sample": f"{reps} x (layer 0's 7 int8 GEMVs + the lm_head GEMV), {sample_bytes} algorithmic "
                          f"bytes in {dt:.1f} s, OpenMP over rows"}
