@@ -719,6 +719,12 @@ Plan make_plan(const GemvCall* calls, int n, int vl) {
         // several batches per wavefront, the same number for all of them (+-1)
         const int per_wave = (first + cap - 1) / cap;
         waves = (first + per_wave - 1) / per_wave;
+        // Long streams: every resident slot gets a wavefront, and the batches that do not divide
+        // evenly go to the lowest-numbered wavefronts.  Those belong to the blocks that reach a
+        // CU first, and the CU serves its oldest wavefronts first: with equal shares they finish
+        // about a microsecond ahead of the second block's and two ahead of the third's (measured
+        // with per-wavefront clocks), so they are the ones that can take one batch more.
+        if (first >= 8L * cap) waves = cap;
         p.pipe = true;
     }
     p.grid = dim3((waves + kWavesPerBlock - 1) / kWavesPerBlock, calls[0].M, 1);
