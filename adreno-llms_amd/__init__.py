@@ -54,6 +54,8 @@ _SIGNATURES = {
     "mi_linear_gate_up_silu": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp]),
     "mi_dequant_int8_to_fp16": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "mi_unpack_q4_to_int8": (_i, [_vp, _vp, _i, _i, _vp]),
+    "mi_argmax_f16": (_i, [_vp, _vp, _i, _i, _vp]),
+    "mi_linear_argmax": (_i, [_vp, _i, _i, _vp, _vp, _vp, _i, _vp]),
     "mi_set_gemm_mode": (None, [_i]),
     "mi_set_gemv_mode": (None, [_i]),
     "mi_quantize_int8": (_i, [_vp, _i, _i, _vp, _vp]),
@@ -266,6 +268,16 @@ def dequant_int8_weight_to_fp16(queue, W_int8, scale_fp16, N, K, out_fp16):
 
 def unpack_q4_to_int8(queue, W_q4, N, K, out_int8):
     return bool(lib().mi_unpack_q4_to_int8(_q(queue), _h(W_q4), N, K, _h(out_int8)))
+
+
+def argmax_f16(queue, logits, N, token_out, num_partials=32):
+    """argmax_partial + argmax_finalize (QW/kernels/gemv_m1.cl:198-280); token_out: int32 on the device."""
+    return bool(lib().mi_argmax_f16(_q(queue), _h(logits), N, num_partials, _h(token_out)))
+
+
+def pytorch_linear_argmax(queue, N, K, x, W, logits, token_out, num_partials=32):
+    """The lm_head of a greedy step: dispatch_lm_head_argmax (QW/src/model.cpp:436-482)."""
+    return bool(lib().mi_linear_argmax(_q(queue), N, K, _h(x), _h(W), _h(logits), num_partials, _h(token_out)))
 
 
 # ------------------------------------------------------------------- offline tools

@@ -56,6 +56,11 @@ bool launch_gate_up_silu(hipStream_t s, WeightKind kind, int N, int K, const voi
 bool launch_dequant_int8(hipStream_t s, const void* q, const void* scale, int N, int K, void* w16);
 bool launch_unpack_q4(hipStream_t s, const void* p, int N, int K, void* w8);
 
+// argmax.hip: index of the greatest of N fp16 values, ties as the reference's two argmax kernels break them.
+// scratch: kArgmaxScratchBytes of device memory that belongs to stream s, or null (then one block does all the work).
+constexpr size_t kArgmaxScratchBytes = 512;
+bool launch_argmax_f16(hipStream_t s, const void* logits, int N, int num_partials, void* token_out, void* scratch);
+
 // gemm.hip: out[M,N] = x[M,K] W^T on MFMA with the dequant fused into the tile load.
 bool gemm_supported(WeightKind kind, int M, int N, int K);
 // workspace: device memory that belongs to stream s (or null): the int8 kernel may cut K into

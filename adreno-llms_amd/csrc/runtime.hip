@@ -244,6 +244,25 @@ int mi_linear(void* stream, int M, int N, int K, const void* x, const void* W, v
     return launch_gemv(as_stream(stream), c) ? 1 : 0;
 }
 
+int mi_argmax_f16(void* stream, const void* logits, int N, int num_partials, void* token_out) {
+    if (!ensure_init()) return 0;
+    if (!logits || !token_out || N <= 0 || num_partials <= 0 || reinterpret_cast<uintptr_t>(logits) % 2 ||
+        reinterpret_cast<uintptr_t>(token_out) % 4) {
+        MI_ERROR_FMT("mi_argmax_f16: bad argument (logits=%p N=%d num_partials=%d token_out=%p)", logits, N,
+                     num_partials, token_out);
+        return 0;
+    }
+    // the stream's workspace doubles as scratch: work on a stream is ordered, and nothing is kept there between calls
+    static_assert(kArgmaxScratchBytes <= kWorkspaceBytes, "scratch fits the workspace");
+    return launch_argmax_f16(as_stream(stream), logits, N, num_partials, token_out, workspace_of(as_stream(stream))) ? 1 : 0;
+}
+
+int mi_linear_argmax(void* stream, int N, int K, const void* x, const void* W, void* logits, int num_partials,
+                     void* token_out) {
+    if (!mi_linear(stream, 1, N, K, x, W, logits)) return 0;
+    return mi_argmax_f16(stream, logits, N, num_partials, token_out);
+}
+
 // True when [a, a+na) and [b, b+nb) share a byte.
 static bool overlaps(const void* a, size_t na, const void* b, size_t nb) {
     const auto pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);

@@ -212,6 +212,15 @@ def main():
         detail["c3_q4_gemv_151936x896"] = cold_gemv("q4", VOCAB, H, 4)
         detail["c3_int8_gemv_151936x896"] = {"us": roofline["us_per_launch"], "GBps": roofline["achieved"],
                                              "frac_hbm": roofline["frac"], "bytes": lm_bytes}
+        # the greedy step's lm_head: GEMV + argmax, token left in device memory
+        token = mil.Buffer(4)
+
+        def lm_head_argmax():
+            for i in range(30):
+                assert mil.pytorch_linear_argmax(queue, VOCAB, H, x_h, copies[i % 3][0], logits, token)
+
+        lm_head_argmax()
+        detail["c4_lm_head_int8_plus_argmax"] = {"us": round(time_region(mil, queue, lm_head_argmax, 5) / 30 * 1e3, 2)}
 
     # ---- config 5: prefill GEMM with fused int8 dequant on the matrix cores ---------------
     if not args.no_detail:

@@ -97,6 +97,23 @@ int mi_dequant_int8_to_fp16(void* stream, const void* W_int8, const void* scale_
  * w8[n,k] = nibble(n,k) - 8 as int8. */
 int mi_unpack_q4_to_int8(void* stream, const void* W_q4, int N, int K, void* w8);
 
+/* Greedy token on the device.  argmax_partial + argmax_finalize (QW/kernels/gemv_m1.cl:198-280, as
+ * enqueued by dispatch_lm_head_argmax, QW/src/model.cpp:436-482, with NUM_PARTIALS = 32 and
+ * work-groups of 64): token_out[0] (one int32 in device memory) = index of the greatest of the N fp16
+ * logits; NaN and -inf never win, no candidate gives 0, and equal maxima are resolved as the two
+ * reference kernels resolve them for the same num_partials (chunks of ceil(N / num_partials) logits;
+ * strict ">" in the strided scans and in the trees makes the smaller bit-reversed work-item number
+ * win: the chunk p with the lowest (bitrev6(p % 64), p), then the lowest
+ * bitrev6((index - chunk start) % 64), then the lowest index).  Two launches on a stream made by
+ * mi_stream_create or the null stream (512 bytes of the stream's workspace take the place of the
+ * reference's two scratch buffers), one slower launch on any other stream.  The token stays on
+ * the device for the next step. */
+int mi_argmax_f16(void* stream, const void* logits, int N, int num_partials, void* token_out);
+/* mi_linear with M = 1 followed by mi_argmax_f16 on its output: the lm_head of a greedy decode step
+ * (QW/src/model.cpp:436-482).  logits [N] fp16 is written as by mi_linear. */
+int mi_linear_argmax(void* stream, int N, int K, const void* x, const void* W, void* logits, int num_partials,
+                     void* token_out);
+
 /* One call of mi_linear, for mi_linear_batch. */
 typedef struct mi_linear_call {
     int M, N, K;

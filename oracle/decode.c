@@ -153,11 +153,12 @@ static void swiglu(uint16_t* gate, const uint16_t* up, int n)
     }
 }
 
-/* argmax_partial with 32 partials of 64 lanes, then argmax_finalize. */
-static int argmax(const uint16_t* x, int N)
+/* argmax_partial with NP partials of 64 lanes, then argmax_finalize
+ * (QW/kernels/gemv_m1.cl:198-280); NP <= 4096. */
+int orc_argmax_f16(const uint16_t* x, int N, int NP)
 {
-    const int NP = 32;
-    float pv[32]; int pi[32];
+    static _Thread_local float pv[4096]; static _Thread_local int pi[4096];
+    if (NP < 1 || NP > 4096 || N < 1) return -1;
     int chunk = (N + NP - 1) / NP;
     for (int wg = 0; wg < NP; ++wg) {
         int start = wg * chunk, end = start + chunk < N ? start + chunk : N;
@@ -261,7 +262,7 @@ int orc_decoder_step(void* p, int token, int pos, orc_linear_fn fn, void* ctx, f
     }
     rmsnorm(d->h, m->final_norm, d->xn, Hd, m->rms_eps);
     linear(d, fn, ctx, m->n_layers * 7, m->vocab, Hd, d->xn, d->logits);
-    int best = argmax(d->logits, m->vocab);
+    int best = orc_argmax_f16(d->logits, m->vocab, 32);
     if (margin) {
         float top = H(d->logits[best]), second = -3.402823466e+38f;
         for (int i = 0; i < m->vocab; ++i)

@@ -88,6 +88,13 @@ void orc_gemm_q4 (const uint16_t* X, const uint8_t* p, const uint16_t* sc, uint1
 
 int orc_max_threads(void);
 
+/* argmax_partial (NP work-groups of 64 over contiguous chunks) + argmax_finalize, literally:
+ * QW/kernels/gemv_m1.cl:198-280.  Index of the greatest fp16 value with the kernels' own tie
+ * behaviour; 1 <= NP <= 4096.  Parity: the tie order is what the source spells out (strict ">" in
+ * the strided scan and in both trees); checked against a brute-force statement of that order in
+ * tests/test_oracle_gemv.py. */
+int orc_argmax_f16(const uint16_t* x, int N, int NP);
+
 #ifdef __cplusplus
 }
 #endif

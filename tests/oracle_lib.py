@@ -46,6 +46,7 @@ def _load():
         "orc_gemm_i8": (None, [_u16p, _i8p, _u16p, _u16p, I, I, I, I]),
         "orc_gemm_q4": (None, [_u16p, _u8p, _u16p, _u16p, I, I, I, I]),
         "orc_max_threads": (I, []),
+        "orc_argmax_f16": (I, [_u16p, I, I]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -130,3 +131,10 @@ def gemm_q4(X, p, sc, threads=THREADS):
     out = np.empty((M, N), np.uint16)
     lib.orc_gemm_q4(u16(X), p, np.ascontiguousarray(sc), out, M, N, K, threads)
     return out
+
+
+def argmax_f16(x, num_partials=32):
+    """x: fp16 values, or their uint16 bit patterns as the gemv_* functions return them."""
+    x = np.asarray(x)
+    x = (np.ascontiguousarray(x) if x.dtype == np.uint16 else u16(x)).reshape(-1)
+    return lib.orc_argmax_f16(x, x.size, num_partials)
