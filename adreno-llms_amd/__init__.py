@@ -54,6 +54,13 @@ _SIGNATURES = {
     "mi_linear_gate_up_silu": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp]),
     "mi_dequant_int8_to_fp16": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "mi_unpack_q4_to_int8": (_i, [_vp, _vp, _i, _i, _vp]),
+    "mi_decoder_create": (_vp, [_vp, _vp]),
+    "mi_decoder_destroy": (_i, [_vp]),
+    "mi_decoder_reset": (_i, [_vp, _vp, _i, _i]),
+    "mi_decoder_set_token": (_i, [_vp, _vp, _i]),
+    "mi_decoder_step": (_i, [_vp, _vp]),
+    "mi_decoder_read": (_i, [_vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
+    "mi_decoder_logits": (_vp, [_vp]),
     "mi_argmax_f16": (_i, [_vp, _vp, _i, _i, _vp]),
     "mi_linear_argmax": (_i, [_vp, _i, _i, _vp, _vp, _vp, _i, _vp]),
     "mi_set_gemm_mode": (None, [_i]),
@@ -278,6 +285,69 @@ def argmax_f16(queue, logits, N, token_out, num_partials=32):
 def pytorch_linear_argmax(queue, N, K, x, W, logits, token_out, num_partials=32):
     """The lm_head of a greedy step: dispatch_lm_head_argmax (QW/src/model.cpp:436-482)."""
     return bool(lib().mi_linear_argmax(_q(queue), N, K, _h(x), _h(W), _h(logits), num_partials, _h(token_out)))
+
+
+class DecoderConfig(C.Structure):
+    """mi_decoder_config (include/mi_decode.h)."""
+    _fields_ = [(n, _i) for n in ("hidden", "inter", "n_heads", "n_kv_heads", "head_dim", "n_layers", "vocab",
+                                  "max_pos")] + [("rms_eps", C.c_float), ("rope_theta", C.c_float)]
+
+
+class DecoderWeights(C.Structure):
+    """mi_decoder_weights (include/mi_decode.h)."""
+    _fields_ = [("embed", _vp), ("final_norm", _vp), ("lm_head", _vp)] + \
+               [(n, C.POINTER(_vp)) for n in ("in_norm", "post_norm", "bq", "bk", "bv", "wq", "wk", "wv", "wo",
+                                              "wgate", "wup", "wdown")]
+
+
+class Decoder:
+    """Greedy decoding on the device (Model::forward_greedy and the decode loop, QW/src/model.cpp:387-500).
+
+    cfg: dict with the DecoderConfig fields; weights: dict name -> Buffer (embed, final_norm, lm_head)
+    or list of Buffers per layer (the other DecoderWeights fields)."""
+
+    def __init__(self, cfg, weights):
+        c = DecoderConfig()
+        for name, _ in DecoderConfig._fields_:
+            setattr(c, name, cfg[name])
+        w = DecoderWeights()
+        self._keep = [weights]
+        for name in ("embed", "final_norm", "lm_head"):
+            setattr(w, name, _h(weights[name]))
+        for name, _ in DecoderWeights._fields_[3:]:
+            arr = (_vp * cfg["n_layers"])(*[_h(b) for b in weights[name]])
+            self._keep.append(arr)
+            setattr(w, name, arr)
+        self.handle = lib().mi_decoder_create(C.byref(c), C.byref(w))
+        if not self.handle:
+            raise RuntimeError("mi_decoder_create failed")
+
+    def reset(self, queue, pos, token):
+        return bool(lib().mi_decoder_reset(self.handle, _q(queue), pos, token))
+
+    def set_token(self, queue, token):
+        return bool(lib().mi_decoder_set_token(self.handle, _q(queue), token))
+
+    def step(self, queue):
+        return bool(lib().mi_decoder_step(self.handle, _q(queue)))
+
+    def read(self, queue):
+        pos, tok = _i(), _i()
+        if not lib().mi_decoder_read(self.handle, _q(queue), C.byref(pos), C.byref(tok)):
+            raise RuntimeError("mi_decoder_read failed")
+        return pos.value, tok.value
+
+    @property
+    def logits_ptr(self):
+        return lib().mi_decoder_logits(self.handle)
+
+    def close(self):
+        if self.handle and _lib is not None:
+            _lib.mi_decoder_destroy(self.handle)
+        self.handle = None
+
+    def __del__(self):
+        self.close()
 
 
 # ------------------------------------------------------------------- offline tools

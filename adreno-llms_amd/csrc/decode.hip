@@ -1,0 +1,386 @@
+// A Qwen2-shaped greedy decode step that stays on the device: the small kernels that sit between
+// the projections (QW/kernels/{embedding,rmsnorm,bias_add,rope,attention,mlp,utils}.cl), the
+// projections themselves through mi_linear / mi_linear_batch, and the argmax.  Graph of a step:
+// QW/src/model.cpp:243-376, QW/src/layers/attention.cpp:336-674, QW/src/layers/mlp.cpp:97-237.
+//
+// Position and token live in device memory (the reference's counter buffer, QW/src/model.cpp:
+// 490-500): every kernel reads them there and the last kernel of a step advances them, so a step
+// is the same sequence of launches with the same arguments at every position: one captured
+// graph replays for the whole generation, and no token returns to the host between steps.
+//
+// These kernels are the harness around the matmul path, not the path: they are written for
+// exactness against the CPU restatement (same operations in the same order, so that the token
+// lists can be compared for identity), and are launch-bound at batch 1 whatever they do.
+#include "common.h"
+#include "device_math.h"
+#include "../../include/mi_decode.h"
+#include "../../include/mi_linear.h"
+
+#include <cmath>
+#include <vector>
+
+namespace mi {
+namespace {
+
+struct State {
+    int pos;
+    int token;
+    int next;       // written by the argmax, moved into token by advance_kernel
+};
+
+__device__ __forceinline__ float rcp_rn(float x) { return __fdiv_rn(1.0f, x); }
+
+// h[c] = embed[token][c]   (QW/kernels/embedding.cl)
+__global__ void embed_kernel(const uint16_t* __restrict__ embed, const State* __restrict__ st,
+                             uint16_t* __restrict__ h, int hidden, int vocab) {
+    int t = st->token;
+    t = t < 0 ? 0 : (t >= vocab ? vocab - 1 : t);
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) h[c] = embed[static_cast<size_t>(t) * hidden + c];
+}
+
+// out[c] = fp16((x[c] * inv) * w[c]), inv = 1 / sqrt(mean(x^2) + eps); the sum of squares runs
+// over 64 work-items in float4 strides and a 32..1 tree (QW/kernels/rmsnorm.cl).  One wavefront.
+__global__ __launch_bounds__(64) void rmsnorm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                     uint16_t* __restrict__ out, int cols, float eps) {
+    const int lid = threadIdx.x, c4n = cols >> 2;
+    float acc = 0.0f;
+    for (int c4 = lid; c4 < c4n; c4 += 64) {
+        const float v0 = h_f(x[4 * c4]), v1 = h_f(x[4 * c4 + 1]), v2 = h_f(x[4 * c4 + 2]), v3 = h_f(x[4 * c4 + 3]);
+        float d = v0 * v0;
+        d = fmaf(v1, v1, d);
+        d = fmaf(v2, v2, d);
+        d = fmaf(v3, v3, d);
+        acc = acc + d;
+    }
+    for (int c = c4n * 4 + lid; c < cols; c += 64) acc = fmaf(h_f(x[c]), h_f(x[c]), acc);
+    #pragma unroll
+    for (int s = 32; s > 0; s >>= 1) {
+        const float o = __shfl_down(acc, s, 64);      // work-item t adds work-item t + s
+        acc = acc + o;
+    }
+    const float total = __shfl(acc, 0, 64);
+    const float inv = rcp_rn(__fsqrt_rn(__fdiv_rn(total, static_cast<float>(cols)) + eps));
+    for (int c = lid; c < cols; c += 64) out[c] = f_h((h_f(x[c]) * inv) * h_f(w[c]));
+}
+
+// a[i] = fp16(a[i] + b[i]) for up to three vectors in one launch (QW/kernels/bias_add.cl, utils.cl)
+struct AddJob {
+    uint16_t* a;
+    const uint16_t* b;
+    int n;
+};
+struct AddJobs {
+    AddJob j[3];
+    int count;
+};
+__global__ void add_kernel(const AddJobs jobs) {
+    for (int k = 0; k < jobs.count; ++k) {
+        const AddJob& j = jobs.j[k];
+        for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < j.n; i += gridDim.x * blockDim.x)
+            j.a[i] = f_h(h_f(j.a[i]) + h_f(j.b[i]));
+    }
+}
+
+// Rotary embedding of q and k at the current position, then k and v into the caches
+// (QW/kernels/rope.cl; cache rows as QW/src/layers/attention.cpp:560-600).
+__global__ void rope_kv_kernel(uint16_t* __restrict__ q, uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
+                               const uint16_t* __restrict__ cosT, const uint16_t* __restrict__ sinT,
+                               uint16_t* __restrict__ kc, uint16_t* __restrict__ vc, const State* __restrict__ st,
+                               int n_heads, int n_kv_heads, int D, int max_pos) {
+    int pos = st->pos;
+    pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+    const int hd2 = D / 2, kvd = n_kv_heads * D;
+    const uint16_t* cr = cosT + static_cast<size_t>(pos) * D;
+    const uint16_t* sr = sinT + static_cast<size_t>(pos) * D;
+    const int pairs = (n_heads + n_kv_heads) * hd2;
+    for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < pairs; p += gridDim.x * blockDim.x) {
+        const int head = p / hd2, i = p % hd2;
+        uint16_t* buf = head < n_heads ? q + head * D : k + (head - n_heads) * D;
+        const float x1 = h_f(buf[i]), x2 = h_f(buf[i + hd2]);
+        const float c = h_f(cr[i]), s = h_f(sr[i]);
+        const float o1 = fmaf(x1, c, -(x2 * s));
+        const float o2 = fmaf(x2, c, x1 * s);
+        const uint16_t r1 = f_h(o1), r2 = f_h(o2);
+        buf[i] = r1;
+        buf[i + hd2] = r2;
+        if (head >= n_heads) {
+            uint16_t* dst = kc + static_cast<size_t>(pos) * kvd + (head - n_heads) * D;
+            dst[i] = r1;
+            dst[i + hd2] = r2;
+        }
+    }
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < kvd; e += gridDim.x * blockDim.x)
+        vc[static_cast<size_t>(pos) * kvd + e] = v[e];
+}
+
+// Single-query grouped-query attention for one head per block (QW/kernels/attention.cl:
+// gqa_attn_scores, gqa_softmax, gqa_attn_out).  Sums run in the order the CPU restatement uses:
+// the score over D in float4 groups, the softmax denominator over the keys in index order, the
+// output over the keys in index order.  Dynamic LDS: max_pos floats.
+__global__ void attention_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc,
+                                 const uint16_t* __restrict__ vc, uint16_t* __restrict__ scores,
+                                 uint16_t* __restrict__ out, const State* __restrict__ st, int n_heads,
+                                 int n_kv_heads, int D, int max_pos, float scale) {
+    extern __shared__ float ex[];
+    __shared__ float red[64];
+    __shared__ float inv_s;
+    int pos = st->pos;
+    pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+    const int seq_k = pos + 1, qh = blockIdx.x, kvd = n_kv_heads * D, kvh = qh / (n_heads / n_kv_heads);
+    const int tid = threadIdx.x, nt = blockDim.x;
+    uint16_t* sc = scores + static_cast<size_t>(qh) * max_pos;
+    const uint16_t* qv = q + qh * D;
+    for (int tk = tid; tk < seq_k; tk += nt) {
+        const uint16_t* kv = kc + static_cast<size_t>(tk) * kvd + kvh * D;
+        float acc = 0.0f;
+        for (int d4 = 0; d4 < D / 4; ++d4) {
+            float t = h_f(qv[4 * d4]) * h_f(kv[4 * d4]);
+            t = fmaf(h_f(qv[4 * d4 + 1]), h_f(kv[4 * d4 + 1]), t);
+            t = fmaf(h_f(qv[4 * d4 + 2]), h_f(kv[4 * d4 + 2]), t);
+            t = fmaf(h_f(qv[4 * d4 + 3]), h_f(kv[4 * d4 + 3]), t);
+            acc = acc + t;
+        }
+        sc[tk] = f_h(acc * scale);
+    }
+    __syncthreads();
+    // maximum (any order gives the same value)
+    float m = -3.402823466e+38f;
+    for (int c = tid; c < seq_k; c += nt) m = fmaxf(m, h_f(sc[c]));
+    if (tid < 64) red[tid] = -3.402823466e+38f;
+    __syncthreads();
+    for (int s = 32; s > 0; s >>= 1) m = fmaxf(m, __shfl_down(m, s, 64));
+    if ((tid & 63) == 0) red[tid >> 6] = m;
+    __syncthreads();
+    float maxv = red[0];
+    for (int i = 1; i < (nt + 63) / 64; ++i) maxv = fmaxf(maxv, red[i]);
+    for (int c = tid; c < seq_k; c += nt) {
+        const float e = exp_poly(h_f(sc[c]) - maxv);
+        ex[c] = e;
+        sc[c] = f_h(e);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        float sum = 0.0f;
+        for (int c = 0; c < seq_k; ++c) sum = sum + ex[c];
+        inv_s = rcp_rn(sum + 1e-20f);
+    }
+    __syncthreads();
+    const float inv = inv_s;
+    for (int c = tid; c < seq_k; c += nt) sc[c] = f_h(h_f(sc[c]) * inv);
+    __syncthreads();
+    for (int e = tid; e < D; e += nt) {
+        float acc = 0.0f;
+        for (int tk = 0; tk < seq_k; ++tk)
+            acc = fmaf(h_f(sc[tk]), h_f(vc[static_cast<size_t>(tk) * kvd + kvh * D + e]), acc);
+        out[qh * D + e] = f_h(acc);
+    }
+}
+
+// gate[i] = fp16((g * sigmoid(g)) * up[i])   (QW/kernels/mlp.cl swiglu_inplace)
+__global__ void swiglu_kernel(uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, int n) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        const float g = h_f(gate[i]), u = h_f(up[i]);
+        const float sig = rcp_rn(1.0f + exp_poly(-g));
+        gate[i] = f_h((g * sig) * u);
+    }
+}
+
+__global__ void advance_kernel(State* st) {
+    st->token = st->next;
+    st->pos = st->pos + 1;
+}
+
+struct Decoder {
+    mi_decoder_config c{};
+    std::vector<const void*> in_norm, post_norm, bq, bk, bv, wq, wk, wv, wo, wgate, wup, wdown;
+    const void* embed = nullptr;
+    const void* final_norm = nullptr;
+    const void* lm_head = nullptr;
+    // device memory owned by the decoder
+    uint16_t *kc = nullptr, *vc = nullptr, *cosT = nullptr, *sinT = nullptr;
+    uint16_t *h = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *proj = nullptr;
+    uint16_t *gate = nullptr, *up = nullptr, *logits = nullptr, *scores = nullptr;
+    State* st = nullptr;
+    std::vector<void*> owned;
+};
+
+template <typename T>
+bool dev_alloc(Decoder* d, T** p, size_t bytes) {
+    void* m = nullptr;
+    if (!MI_HIP_OK(hipMalloc(&m, bytes ? bytes : 1))) return false;
+    d->owned.push_back(m);
+    *p = static_cast<T*>(m);
+    return true;
+}
+
+uint16_t host_f16(float f) { return mi_f32_to_f16(f); }
+
+}  // namespace
+}  // namespace mi
+
+using namespace mi;
+
+extern "C" {
+
+void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* w) {
+    if (!cfg || !w || mi_init(0) != 1) return nullptr;
+    const mi_decoder_config& c = *cfg;
+    if (c.hidden <= 0 || c.inter <= 0 || c.n_heads <= 0 || c.n_kv_heads <= 0 || c.head_dim <= 0 || c.n_layers <= 0 ||
+        c.vocab <= 0 || c.max_pos <= 0 || c.n_heads % c.n_kv_heads || c.head_dim % 4 || c.max_pos > 8192) {
+        MI_ERROR_FMT("mi_decoder_create: bad configuration");
+        return nullptr;
+    }
+    auto* d = new Decoder;
+    d->c = c;
+    const int L = c.n_layers;
+    auto take = [L](std::vector<const void*>& dst, const void* const* src) {
+        dst.assign(src, src + L);
+    };
+    take(d->in_norm, w->in_norm); take(d->post_norm, w->post_norm);
+    take(d->bq, w->bq); take(d->bk, w->bk); take(d->bv, w->bv);
+    take(d->wq, w->wq); take(d->wk, w->wk); take(d->wv, w->wv); take(d->wo, w->wo);
+    take(d->wgate, w->wgate); take(d->wup, w->wup); take(d->wdown, w->wdown);
+    d->embed = w->embed; d->final_norm = w->final_norm; d->lm_head = w->lm_head;
+
+    const int D = c.head_dim, kvd = c.n_kv_heads * D, qd = c.n_heads * D;
+    const size_t cache = static_cast<size_t>(L) * c.max_pos * kvd * 2;
+    bool ok = dev_alloc(d, &d->kc, cache) && dev_alloc(d, &d->vc, cache) &&
+              dev_alloc(d, &d->cosT, static_cast<size_t>(c.max_pos) * D * 2) &&
+              dev_alloc(d, &d->sinT, static_cast<size_t>(c.max_pos) * D * 2) &&
+              dev_alloc(d, &d->h, c.hidden * 2) && dev_alloc(d, &d->xn, c.hidden * 2) && dev_alloc(d, &d->q, qd * 2) &&
+              dev_alloc(d, &d->k, kvd * 2) && dev_alloc(d, &d->v, kvd * 2) && dev_alloc(d, &d->attn, qd * 2) &&
+              dev_alloc(d, &d->proj, c.hidden * 2) && dev_alloc(d, &d->gate, c.inter * 2) &&
+              dev_alloc(d, &d->up, c.inter * 2) && dev_alloc(d, &d->logits, static_cast<size_t>(c.vocab) * 2) &&
+              dev_alloc(d, &d->scores, static_cast<size_t>(c.n_heads) * c.max_pos * 2) &&
+              dev_alloc(d, &d->st, sizeof(State));
+    if (ok) {
+        // rotary tables, QW/src/layers/attention.cpp:133-172: cos/sin(t * theta^(-2i/D)), both halves alike
+        std::vector<uint16_t> ct(static_cast<size_t>(c.max_pos) * D), stb(ct.size());
+        for (int t = 0; t < c.max_pos; ++t)
+            for (int i = 0; i < D / 2; ++i) {
+                const float exponent = (2.0f * static_cast<float>(i)) / static_cast<float>(D);
+                const float inv_freq = powf(c.rope_theta, -exponent);
+                const float angle = static_cast<float>(t) * inv_freq;
+                const uint16_t cv = host_f16(cosf(angle)), sv = host_f16(sinf(angle));
+                ct[static_cast<size_t>(t) * D + i] = cv; ct[static_cast<size_t>(t) * D + i + D / 2] = cv;
+                stb[static_cast<size_t>(t) * D + i] = sv; stb[static_cast<size_t>(t) * D + i + D / 2] = sv;
+            }
+        const State zero{0, 0, 0};
+        ok = MI_HIP_OK(hipMemcpy(d->cosT, ct.data(), ct.size() * 2, hipMemcpyHostToDevice)) &&
+             MI_HIP_OK(hipMemcpy(d->sinT, stb.data(), stb.size() * 2, hipMemcpyHostToDevice)) &&
+             MI_HIP_OK(hipMemset(d->kc, 0, cache)) && MI_HIP_OK(hipMemset(d->vc, 0, cache)) &&
+             MI_HIP_OK(hipMemcpy(d->st, &zero, sizeof zero, hipMemcpyHostToDevice));
+    }
+    if (!ok) {
+        mi_decoder_destroy(d);
+        return nullptr;
+    }
+    return d;
+}
+
+int mi_decoder_destroy(void* dec) {
+    auto* d = static_cast<Decoder*>(dec);
+    if (!d) return 1;
+    for (void* p : d->owned) (void)hipFree(p);
+    delete d;
+    return 1;
+}
+
+int mi_decoder_reset(void* dec, void* stream, int pos, int token) {
+    auto* d = static_cast<Decoder*>(dec);
+    if (!d || pos < 0 || pos >= d->c.max_pos || token < 0 || token >= d->c.vocab) {
+        MI_ERROR_FMT("mi_decoder_reset: bad argument (pos=%d token=%d)", pos, token);
+        return 0;
+    }
+    const State s{pos, token, token};
+    auto st = static_cast<hipStream_t>(stream);
+    return MI_HIP_OK(hipMemcpyAsync(d->st, &s, sizeof s, hipMemcpyHostToDevice, st)) && MI_HIP_OK(hipStreamSynchronize(st));
+}
+
+int mi_decoder_set_token(void* dec, void* stream, int token) {
+    auto* d = static_cast<Decoder*>(dec);
+    if (!d || token < 0 || token >= d->c.vocab) {
+        MI_ERROR_FMT("mi_decoder_set_token: bad argument (token=%d)", token);
+        return 0;
+    }
+    auto st = static_cast<hipStream_t>(stream);
+    return MI_HIP_OK(hipMemcpyAsync(reinterpret_cast<char*>(d->st) + offsetof(State, token), &token, sizeof token,
+                                    hipMemcpyHostToDevice, st)) && MI_HIP_OK(hipStreamSynchronize(st));
+}
+
+int mi_decoder_read(void* dec, void* stream, int* pos, int* token) {
+    auto* d = static_cast<Decoder*>(dec);
+    if (!d) return 0;
+    State s{};
+    auto st = static_cast<hipStream_t>(stream);
+    if (!MI_HIP_OK(hipMemcpyAsync(&s, d->st, sizeof s, hipMemcpyDeviceToHost, st)) || !MI_HIP_OK(hipStreamSynchronize(st)))
+        return 0;
+    if (pos) *pos = s.pos;
+    if (token) *token = s.token;
+    return 1;
+}
+
+const void* mi_decoder_logits(void* dec) { return dec ? static_cast<Decoder*>(dec)->logits : nullptr; }
+
+int mi_decoder_step(void* dec, void* stream) {
+    auto* d = static_cast<Decoder*>(dec);
+    if (!d) return 0;
+    const mi_decoder_config& c = d->c;
+    auto s = static_cast<hipStream_t>(stream);
+    const int Hd = c.hidden, D = c.head_dim, qd = c.n_heads * D, kvd = c.n_kv_heads * D;
+    const float scale = 1.0f / sqrtf(static_cast<float>(D));
+    auto launched = [] { return MI_HIP_OK(hipGetLastError()); };
+    auto rmsnorm = [&](const uint16_t* x, const void* w, uint16_t* out) {
+        hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(64), 0, s, x, static_cast<const uint16_t*>(w), out, Hd, c.rms_eps);
+        return launched();
+    };
+    auto add = [&](const AddJobs& jobs, int nmax) {
+        hipLaunchKernelGGL(add_kernel, dim3((nmax + 255) / 256), dim3(256), 0, s, jobs);
+        return launched();
+    };
+    hipLaunchKernelGGL(embed_kernel, dim3(1), dim3(256), 0, s, static_cast<const uint16_t*>(d->embed), d->st, d->h, Hd, c.vocab);
+    if (!launched()) return 0;
+    for (int l = 0; l < c.n_layers; ++l) {
+        if (!rmsnorm(d->h, d->in_norm[l], d->xn)) return 0;
+        const mi_linear_call qkv[3] = {{1, qd, Hd, d->xn, d->wq[l], d->q},
+                                       {1, kvd, Hd, d->xn, d->wk[l], d->k},
+                                       {1, kvd, Hd, d->xn, d->wv[l], d->v}};
+        if (mi_linear_batch(stream, qkv, 3) != 3) return 0;
+        AddJobs bias{};
+        bias.j[0] = {d->q, static_cast<const uint16_t*>(d->bq[l]), qd};
+        bias.j[1] = {d->k, static_cast<const uint16_t*>(d->bk[l]), kvd};
+        bias.j[2] = {d->v, static_cast<const uint16_t*>(d->bv[l]), kvd};
+        bias.count = 3;
+        if (!add(bias, qd)) return 0;
+        uint16_t* kc = d->kc + static_cast<size_t>(l) * c.max_pos * kvd;
+        uint16_t* vc = d->vc + static_cast<size_t>(l) * c.max_pos * kvd;
+        const int pairs = (c.n_heads + c.n_kv_heads) * D / 2;
+        hipLaunchKernelGGL(rope_kv_kernel, dim3((pairs + 255) / 256), dim3(256), 0, s, d->q, d->k, d->v, d->cosT, d->sinT,
+                           kc, vc, d->st, c.n_heads, c.n_kv_heads, D, c.max_pos);
+        if (!launched()) return 0;
+        const int at = D > 64 ? D : 64;
+        hipLaunchKernelGGL(attention_kernel, dim3(c.n_heads), dim3(at), static_cast<size_t>(c.max_pos) * 4, s, d->q, kc, vc,
+                           d->scores, d->attn, d->st, c.n_heads, c.n_kv_heads, D, c.max_pos, scale);
+        if (!launched()) return 0;
+        if (!mi_linear(stream, 1, Hd, qd, d->attn, d->wo[l], d->proj)) return 0;
+        AddJobs res{};
+        res.j[0] = {d->h, d->proj, Hd};
+        res.count = 1;
+        if (!add(res, Hd)) return 0;
+        if (!rmsnorm(d->h, d->post_norm[l], d->xn)) return 0;
+        const mi_linear_call gu[2] = {{1, c.inter, Hd, d->xn, d->wgate[l], d->gate}, {1, c.inter, Hd, d->xn, d->wup[l], d->up}};
+        if (mi_linear_batch(stream, gu, 2) != 2) return 0;
+        hipLaunchKernelGGL(swiglu_kernel, dim3((c.inter + 255) / 256), dim3(256), 0, s, d->gate, d->up, c.inter);
+        if (!launched()) return 0;
+        if (!mi_linear(stream, 1, Hd, c.inter, d->gate, d->wdown[l], d->proj)) return 0;
+        if (!add(res, Hd)) return 0;
+    }
+    if (!rmsnorm(d->h, d->final_norm, d->xn)) return 0;
+    if (!mi_linear_argmax(stream, c.vocab, Hd, d->xn, d->lm_head, d->logits, 32,
+                          reinterpret_cast<char*>(d->st) + offsetof(State, next)))
+        return 0;
+    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->st);
+    return launched() ? 1 : 0;
+}
+
+}  // extern "C"

@@ -102,10 +102,12 @@ def main():
     logits = mil.Buffer(VOCAB * 2)
     sweep_bytes = 0
     host_layer0 = {}
+    layer_w = [dict() for _ in range(LAYERS)]
     for layer in range(LAYERS):
         for j, (name, N, K) in enumerate(LAYER_SHAPES):
             qb, sb, host = make_i8(1000 + layer * 16 + j, N, K)
             keep += [qb, sb]
+            layer_w[layer][name] = qb
             if layer == 0:
                 host_layer0[name] = host
             cur, nxt = hidden[layer % 2], hidden[(layer + 1) % 2]
@@ -221,6 +223,38 @@ def main():
 
         lm_head_argmax()
         detail["c4_lm_head_int8_plus_argmax"] = {"us": round(time_region(mil, queue, lm_head_argmax, 5) / 30 * 1e3, 2)}
+
+    # ---- config 4, whole step: every kernel of a greedy decode step on the device -----------
+    if not args.no_detail and not args.no_graph:
+        one = np.float16(1.0)
+        vec = lambda seed, n, base=0.0: mil.Buffer.from_host(np.float16(base) + mil.synth_normal_f16(seed, 0.02, (n,)))
+        QD, KVD = 14 * 64, 2 * 64
+        dec_w = dict(embed=mil.Buffer.from_host(mil.synth_normal_f16(5000, 0.02, (VOCAB, H))),
+                     final_norm=vec(5001, H, 1.0), lm_head=lm_q,
+                     in_norm=[vec(5100 + l, H, 1.0) for l in range(LAYERS)],
+                     post_norm=[vec(5200 + l, H, 1.0) for l in range(LAYERS)],
+                     bq=[vec(5300 + l, QD) for l in range(LAYERS)], bk=[vec(5400 + l, KVD) for l in range(LAYERS)],
+                     bv=[vec(5500 + l, KVD) for l in range(LAYERS)])
+        for key, name in (("wq", "q"), ("wk", "k"), ("wv", "v"), ("wo", "o"), ("wgate", "gate"), ("wup", "up"),
+                          ("wdown", "down")):
+            dec_w[key] = [layer_w[l][name] for l in range(LAYERS)]
+        cfg = dict(hidden=H, inter=INTER, n_heads=14, n_kv_heads=2, head_dim=64, n_layers=LAYERS, vocab=VOCAB,
+                   max_pos=512, rms_eps=1e-6, rope_theta=1000000.0)
+        dec = mil.Decoder(cfg, dec_w)
+        assert dec.reset(queue, 0, 785)
+        assert dec.step(queue)
+        queue.finish()
+        assert dec.reset(queue, 0, 785)
+        with mil.Graph(queue) as step_graph:
+            assert dec.step(queue)
+        for _ in range(8):
+            step_graph.launch()
+        ms_tok = time_region(mil, queue, step_graph.launch, 64)
+        pos_after, _ = dec.read(queue)
+        detail["c4_whole_decode_step_on_device"] = {
+            "us_per_token": round(ms_tok * 1e3, 1), "tokens_per_s": round(1e3 / ms_tok, 1),
+            "launches_per_step": 24 * 12 + 5, "positions": f"8..{pos_after - 1}", "launch": "hip_graph"}
+        dec.close()
 
     # ---- config 5: prefill GEMM with fused int8 dequant on the matrix cores ---------------
     if not args.no_detail:

@@ -1,0 +1,74 @@
+/* mi_decode.h - a greedy decode step of a Qwen2-shaped model that stays on the device.
+ *
+ * The projections and the lm_head go through mi_linear / mi_linear_batch / mi_linear_argmax
+ * (mi_linear.h); this header adds the harness around them that a decode loop needs to run without
+ * the host: embedding lookup, RMSNorm, q/k/v bias, rotary embedding + KV-cache write, single-query
+ * grouped-query attention, SwiGLU, residual adds.  It stands for Model::forward_greedy and the
+ * decode loop of QW/src/model.cpp:243-376, 387-500, 709-856 with QW/src/layers/attention.cpp:336-674
+ * and QW/src/layers/mlp.cpp:97-237, restricted to batch 1, one new token per step.
+ *
+ * Position and token are device state (the reference keeps {start_pos, seq_k} in a counter buffer
+ * read by the kernels, QW/src/model.cpp:490-500): mi_decoder_step enqueues the same launches with
+ * the same arguments at every position, so it can be captured once (mi_graph_begin / mi_graph_end)
+ * and replayed for every token.
+ */
+#ifndef MI_DECODE_H
+#define MI_DECODE_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* MODEL_CONFIG of QW/src/model_config.h:12-34. */
+typedef struct mi_decoder_config {
+    int hidden, inter, n_heads, n_kv_heads, head_dim, n_layers, vocab, max_pos;
+    float rms_eps, rope_theta;
+} mi_decoder_config;
+
+/* Device pointers, caller-owned, alive as long as the decoder.  Norm weights and biases are fp16
+ * vectors; embed is fp16 [vocab, hidden]; projection weights are fp16 [N, K] or quantised and
+ * registered (mi_register_int8_weight / mi_register_q4_weight).  Arrays have n_layers entries. */
+typedef struct mi_decoder_weights {
+    const void* embed;
+    const void* final_norm;
+    const void* lm_head;                 /* [vocab, hidden] */
+    const void* const* in_norm;          /* input_layernorm          [hidden] */
+    const void* const* post_norm;        /* post_attention_layernorm [hidden] */
+    const void* const* bq;               /* [n_heads * head_dim] */
+    const void* const* bk;               /* [n_kv_heads * head_dim] */
+    const void* const* bv;
+    const void* const* wq;               /* [n_heads * head_dim, hidden] */
+    const void* const* wk;               /* [n_kv_heads * head_dim, hidden] */
+    const void* const* wv;
+    const void* const* wo;               /* [hidden, n_heads * head_dim] */
+    const void* const* wgate;            /* [inter, hidden] */
+    const void* const* wup;
+    const void* const* wdown;            /* [hidden, inter] */
+} mi_decoder_weights;
+
+/* Allocates the KV caches ([n_layers, max_pos, n_kv_heads * head_dim] fp16 each), the activation
+ * buffers, the rotary tables (QW/src/layers/attention.cpp:133-172) and the device state
+ * (position 0, token 0).  max_pos <= 8192.  NULL on failure. */
+void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* weights);
+int   mi_decoder_destroy(void* decoder);
+
+/* Device state := {pos, token}; synchronises the stream.  The KV cache rows below pos are kept. */
+int   mi_decoder_reset(void* decoder, void* stream, int pos, int token);
+/* Overrides the token the next step consumes (prompt feeding); synchronises the stream. */
+int   mi_decoder_set_token(void* decoder, void* stream, int token);
+
+/* Enqueues one step: consumes the device token at the device position, writes the KV rows of that
+ * position, leaves the greedy next token as the device token and advances the position.  Nothing is
+ * allocated or synchronised; may be captured into a graph.  A step at position max_pos - 1 is the
+ * last valid one (later steps clamp the position and overwrite that row). */
+int   mi_decoder_step(void* decoder, void* stream);
+
+/* Reads the device state back (synchronises the stream). */
+int   mi_decoder_read(void* decoder, void* stream, int* pos, int* token);
+/* fp16 [vocab] logits of the last step, in device memory. */
+const void* mi_decoder_logits(void* decoder);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

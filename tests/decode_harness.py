@@ -139,3 +139,50 @@ class GpuLinear:
     def close(self):
         for w in self.W:
             mil.nnopt_unregister_weight(w)
+
+
+class GpuDecoder:
+    """The whole step on the device (mi_decoder_*): weights uploaded once, tokens read back only
+    to build the list that is compared."""
+
+    def __init__(self, model, queue):
+        c = model.cfg
+        self.model, self.queue = model, queue
+        self.W = [mil.Buffer.from_host(q) for q in model.w8]
+        self.S = [mil.Buffer.from_host(s) for s in model.ws]
+        for (N, K), w, s in zip(model.shapes, self.W, self.S):
+            assert mil.nnopt_register_int8_weight(w, s, N, K)
+        up = lambda arrs: [mil.Buffer.from_host(a) for a in arrs]
+        L = c["n_layers"]
+        self.bufs = dict(embed=mil.Buffer.from_host(model.embed), final_norm=mil.Buffer.from_host(model.final_norm),
+                         lm_head=self.W[-1], in_norm=up(model.in_norm), post_norm=up(model.post_norm),
+                         bq=up(model.bq), bk=up(model.bk), bv=up(model.bv))
+        for j, name in enumerate(("wq", "wk", "wv", "wo", "wgate", "wup", "wdown")):
+            self.bufs[name] = [self.W[l * 7 + j] for l in range(L)]
+        self.dec = mil.Decoder(c, self.bufs)
+
+    def greedy(self, prompt, n_new, graph=False):
+        q, d = self.queue, self.dec
+        vocab = self.model.cfg["vocab"]
+        assert d.reset(q, 0, int(prompt[0]) % vocab)
+        g = None
+        if graph:
+            d.step(q)                                # warm-up outside the capture (first-use setup of the kernels)
+            q.finish()
+            assert d.reset(q, 0, int(prompt[0]) % vocab)
+            with mil.Graph(q) as g:
+                assert d.step(q)
+        run = (lambda: g.launch()) if graph else (lambda: d.step(q))
+        for t in prompt[1:]:
+            run()
+            assert d.set_token(q, int(t) % vocab)    # prompt feeding: the model's own prediction is overridden
+        toks = []
+        for _ in range(n_new):
+            run()
+            toks.append(d.read(q)[1])
+        return toks
+
+    def close(self):
+        self.dec.close()
+        for w in self.W:
+            mil.nnopt_unregister_weight(w)

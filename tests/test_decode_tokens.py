@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as O
-from decode_harness import PROMPT, QWEN25_05B, TINY, GpuLinear, Model, greedy
+from decode_harness import PROMPT, QWEN25_05B, TINY, GpuDecoder, GpuLinear, Model, greedy
 from helpers import mil
 
 
@@ -60,3 +60,37 @@ def test_qwen_shaped_32_greedy_tokens_identical_on_gpu():
     print("tokens", got, "min top-1/top-2 margin", min(margins), flush=True)
     assert got == want
     assert len(set(got)) > 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("graph", [False, True], ids=["stream", "graph"])
+def test_tiny_model_whole_step_on_device(graph):
+    """mi_decoder_*: every kernel of the step on the GPU, tokens chained in device memory; the token
+    list equals the CPU harness's (the small kernels repeat its operations in its order)."""
+    assert mil.lib().mi_init(0) == 1
+    mil.lib().mi_set_gemv_mode(0)
+    try:
+        queue = mil.Queue()
+        m = Model(TINY, seed=11)
+        want, _ = greedy(m, PROMPT, 32)
+        gd = GpuDecoder(m, queue)
+        got = gd.greedy(PROMPT, 32, graph=graph)
+        gd.close()
+        assert got == want
+    finally:
+        mil.lib().mi_set_gemv_mode(1)
+
+
+@pytest.mark.gpu
+def test_qwen_shaped_whole_step_on_device_graph_replay():
+    assert mil.lib().mi_init(0) == 1
+    queue = mil.Queue()
+    m = Model(QWEN25_05B, seed=2024)
+    want, _ = greedy(m, PROMPT, 32)
+    gd = GpuDecoder(m, queue)
+    got = gd.greedy(PROMPT, 32, graph=True)
+    pos, _ = gd.dec.read(queue)
+    gd.close()
+    print("tokens", got, flush=True)
+    assert got == want
+    assert pos == len(PROMPT) - 1 + 32       # the first prompt token is set by reset, every later token costs a step
