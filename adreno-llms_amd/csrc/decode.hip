@@ -40,19 +40,72 @@ __global__ void embed_kernel(const uint16_t* __restrict__ embed, const State* __
 
 // out[c] = fp16((x[c] * inv) * w[c]), inv = 1 / sqrt(mean(x^2) + eps); the sum of squares runs
 // over 64 work-items in float4 strides and a 32..1 tree (QW/kernels/rmsnorm.cl).  One wavefront.
-__global__ __launch_bounds__(64) void rmsnorm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
-                                                     uint16_t* __restrict__ out, int cols, float eps) {
+// With add != null the residual add that precedes the norm in the step runs first, in the same
+// launch: x[c] = fp16(x[c] + add[c]) (QW/kernels/utils.cl element_add), then the norm of the
+// rounded x, exactly as two launches would compute it.
+__global__ __launch_bounds__(64) void rmsnorm_kernel(uint16_t* __restrict__ x, const uint16_t* __restrict__ add,
+                                                     const uint16_t* __restrict__ w, uint16_t* __restrict__ out,
+                                                     int cols, float eps) {
+    // Work-item lid owns the float4 groups lid, lid + 64, ...: it adds, squares and normalises the
+    // same elements, so x, add and w are read once, all loads are in flight together, and the
+    // kernel costs one memory round trip.  Up to kGroups groups per work-item live in registers
+    // (cols <= 256 kGroups); the tail that is not a whole group, and longer rows, go through memory.
+    constexpr int kGroups = 8;
     const int lid = threadIdx.x, c4n = cols >> 2;
+    typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+    u16x4 xv[kGroups], wv[kGroups];
     float acc = 0.0f;
-    for (int c4 = lid; c4 < c4n; c4 += 64) {
-        const float v0 = h_f(x[4 * c4]), v1 = h_f(x[4 * c4 + 1]), v2 = h_f(x[4 * c4 + 2]), v3 = h_f(x[4 * c4 + 3]);
-        float d = v0 * v0;
-        d = fmaf(v1, v1, d);
-        d = fmaf(v2, v2, d);
-        d = fmaf(v3, v3, d);
+    #pragma unroll
+    for (int g = 0; g < kGroups; ++g) {
+        const int c4 = lid + 64 * g;
+        if (c4 < c4n) {
+            xv[g] = *reinterpret_cast<const u16x4*>(x + 4 * c4);
+            wv[g] = *reinterpret_cast<const u16x4*>(w + 4 * c4);
+            if (add) {
+                const u16x4 av = *reinterpret_cast<const u16x4*>(add + 4 * c4);
+                #pragma unroll
+                for (int e = 0; e < 4; ++e) xv[g][e] = f_h(h_f(xv[g][e]) + h_f(av[e]));
+                *reinterpret_cast<u16x4*>(x + 4 * c4) = xv[g];
+            }
+        }
+    }
+    #pragma unroll
+    for (int g = 0; g < kGroups; ++g) {
+        if (lid + 64 * g < c4n) {
+            const float v0 = h_f(xv[g][0]), v1 = h_f(xv[g][1]), v2 = h_f(xv[g][2]), v3 = h_f(xv[g][3]);
+            float d = v0 * v0;
+            d = fmaf(v1, v1, d);
+            d = fmaf(v2, v2, d);
+            d = fmaf(v3, v3, d);
+            acc = acc + d;
+        }
+    }
+    for (int c4 = lid + 64 * kGroups; c4 < c4n; c4 += 64) {           // rows longer than the registers hold
+        float v[4];
+        #pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[e] = h_f(x[4 * c4 + e]);
+            if (add) {
+                const uint16_t r = f_h(v[e] + h_f(add[4 * c4 + e]));
+                x[4 * c4 + e] = r;
+                v[e] = h_f(r);
+            }
+        }
+        float d = v[0] * v[0];
+        d = fmaf(v[1], v[1], d);
+        d = fmaf(v[2], v[2], d);
+        d = fmaf(v[3], v[3], d);
         acc = acc + d;
     }
-    for (int c = c4n * 4 + lid; c < cols; c += 64) acc = fmaf(h_f(x[c]), h_f(x[c]), acc);
+    for (int c = c4n * 4 + lid; c < cols; c += 64) {                    // cols not a multiple of 4
+        float v = h_f(x[c]);
+        if (add) {
+            const uint16_t r = f_h(v + h_f(add[c]));
+            x[c] = r;
+            v = h_f(r);
+        }
+        acc = fmaf(v, v, acc);
+    }
     #pragma unroll
     for (int s = 32; s > 0; s >>= 1) {
         const float o = __shfl_down(acc, s, 64);      // work-item t adds work-item t + s
@@ -60,33 +113,30 @@ __global__ __launch_bounds__(64) void rmsnorm_kernel(const uint16_t* __restrict_
     }
     const float total = __shfl(acc, 0, 64);
     const float inv = rcp_rn(__fsqrt_rn(__fdiv_rn(total, static_cast<float>(cols)) + eps));
-    for (int c = lid; c < cols; c += 64) out[c] = f_h((h_f(x[c]) * inv) * h_f(w[c]));
-}
-
-// a[i] = fp16(a[i] + b[i]) for up to three vectors in one launch (QW/kernels/bias_add.cl, utils.cl)
-struct AddJob {
-    uint16_t* a;
-    const uint16_t* b;
-    int n;
-};
-struct AddJobs {
-    AddJob j[3];
-    int count;
-};
-__global__ void add_kernel(const AddJobs jobs) {
-    for (int k = 0; k < jobs.count; ++k) {
-        const AddJob& j = jobs.j[k];
-        for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < j.n; i += gridDim.x * blockDim.x)
-            j.a[i] = f_h(h_f(j.a[i]) + h_f(j.b[i]));
+    #pragma unroll
+    for (int g = 0; g < kGroups; ++g) {
+        const int c4 = lid + 64 * g;
+        if (c4 < c4n) {
+            u16x4 o;
+            #pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = f_h((h_f(xv[g][e]) * inv) * h_f(wv[g][e]));
+            *reinterpret_cast<u16x4*>(out + 4 * c4) = o;
+        }
     }
+    for (int c4 = lid + 64 * kGroups; c4 < c4n; c4 += 64)
+        for (int e = 0; e < 4; ++e) out[4 * c4 + e] = f_h((h_f(x[4 * c4 + e]) * inv) * h_f(w[4 * c4 + e]));
+    for (int c = c4n * 4 + lid; c < cols; c += 64) out[c] = f_h((h_f(x[c]) * inv) * h_f(w[c]));
 }
 
-// Rotary embedding of q and k at the current position, then k and v into the caches
-// (QW/kernels/rope.cl; cache rows as QW/src/layers/attention.cpp:560-600).
-__global__ void rope_kv_kernel(uint16_t* __restrict__ q, uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
-                               const uint16_t* __restrict__ cosT, const uint16_t* __restrict__ sinT,
-                               uint16_t* __restrict__ kc, uint16_t* __restrict__ vc, const State* __restrict__ st,
-                               int n_heads, int n_kv_heads, int D, int max_pos) {
+// q/k/v bias (QW/kernels/bias_add.cl), rotary embedding of q and k at the current position
+// (QW/kernels/rope.cl), then k and v into the caches (rows as QW/src/layers/attention.cpp:560-600):
+// one launch, each value rounded to fp16 where the separate kernels would store it.
+__global__ void bias_rope_kv_kernel(uint16_t* __restrict__ q, uint16_t* __restrict__ k, uint16_t* __restrict__ v,
+                                    const uint16_t* __restrict__ bq, const uint16_t* __restrict__ bk,
+                                    const uint16_t* __restrict__ bv, const uint16_t* __restrict__ cosT,
+                                    const uint16_t* __restrict__ sinT, uint16_t* __restrict__ kc,
+                                    uint16_t* __restrict__ vc, const State* __restrict__ st, int n_heads,
+                                    int n_kv_heads, int D, int max_pos) {
     int pos = st->pos;
     pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
     const int hd2 = D / 2, kvd = n_kv_heads * D;
@@ -96,7 +146,9 @@ __global__ void rope_kv_kernel(uint16_t* __restrict__ q, uint16_t* __restrict__ 
     for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < pairs; p += gridDim.x * blockDim.x) {
         const int head = p / hd2, i = p % hd2;
         uint16_t* buf = head < n_heads ? q + head * D : k + (head - n_heads) * D;
-        const float x1 = h_f(buf[i]), x2 = h_f(buf[i + hd2]);
+        const uint16_t* bias = head < n_heads ? bq + head * D : bk + (head - n_heads) * D;
+        const float x1 = h_f(f_h(h_f(buf[i]) + h_f(bias[i])));
+        const float x2 = h_f(f_h(h_f(buf[i + hd2]) + h_f(bias[i + hd2])));
         const float c = h_f(cr[i]), s = h_f(sr[i]);
         const float o1 = fmaf(x1, c, -(x2 * s));
         const float o2 = fmaf(x2, c, x1 * s);
@@ -109,26 +161,30 @@ __global__ void rope_kv_kernel(uint16_t* __restrict__ q, uint16_t* __restrict__ 
             dst[i + hd2] = r2;
         }
     }
-    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < kvd; e += gridDim.x * blockDim.x)
-        vc[static_cast<size_t>(pos) * kvd + e] = v[e];
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < kvd; e += gridDim.x * blockDim.x) {
+        const uint16_t r = f_h(h_f(v[e]) + h_f(bv[e]));
+        v[e] = r;
+        vc[static_cast<size_t>(pos) * kvd + e] = r;
+    }
 }
 
 // Single-query grouped-query attention for one head per block (QW/kernels/attention.cl:
 // gqa_attn_scores, gqa_softmax, gqa_attn_out).  Sums run in the order the CPU restatement uses:
 // the score over D in float4 groups, the softmax denominator over the keys in index order, the
-// output over the keys in index order.  Dynamic LDS: max_pos floats.
+// output over the keys in index order.  The scores (fp16, as the reference's score buffer holds
+// them) and the fp32 exponentials stay in LDS: dynamic LDS of 6 bytes per position.
 __global__ void attention_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc,
-                                 const uint16_t* __restrict__ vc, uint16_t* __restrict__ scores,
-                                 uint16_t* __restrict__ out, const State* __restrict__ st, int n_heads,
-                                 int n_kv_heads, int D, int max_pos, float scale) {
+                                 const uint16_t* __restrict__ vc, uint16_t* __restrict__ out,
+                                 const State* __restrict__ st, int n_heads, int n_kv_heads, int D, int max_pos,
+                                 float scale) {
     extern __shared__ float ex[];
+    uint16_t* sc = reinterpret_cast<uint16_t*>(ex + max_pos);
     __shared__ float red[64];
     __shared__ float inv_s;
     int pos = st->pos;
     pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
     const int seq_k = pos + 1, qh = blockIdx.x, kvd = n_kv_heads * D, kvh = qh / (n_heads / n_kv_heads);
     const int tid = threadIdx.x, nt = blockDim.x;
-    uint16_t* sc = scores + static_cast<size_t>(qh) * max_pos;
     const uint16_t* qv = q + qh * D;
     for (int tk = tid; tk < seq_k; tk += nt) {
         const uint16_t* kv = kc + static_cast<size_t>(tk) * kvd + kvh * D;
@@ -199,7 +255,7 @@ struct Decoder {
     // device memory owned by the decoder
     uint16_t *kc = nullptr, *vc = nullptr, *cosT = nullptr, *sinT = nullptr;
     uint16_t *h = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *proj = nullptr;
-    uint16_t *gate = nullptr, *up = nullptr, *logits = nullptr, *scores = nullptr;
+    uint16_t *gate = nullptr, *up = nullptr, *logits = nullptr;
     State* st = nullptr;
     std::vector<void*> owned;
 };
@@ -241,6 +297,15 @@ void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* 
     take(d->wq, w->wq); take(d->wk, w->wk); take(d->wv, w->wv); take(d->wo, w->wo);
     take(d->wgate, w->wgate); take(d->wup, w->wup); take(d->wdown, w->wdown);
     d->embed = w->embed; d->final_norm = w->final_norm; d->lm_head = w->lm_head;
+    bool aligned = reinterpret_cast<uintptr_t>(w->final_norm) % 8 == 0;
+    for (int l = 0; l < L; ++l)
+        aligned = aligned && reinterpret_cast<uintptr_t>(w->in_norm[l]) % 8 == 0 &&
+                  reinterpret_cast<uintptr_t>(w->post_norm[l]) % 8 == 0;
+    if (!aligned || c.hidden % 4) {
+        MI_ERROR_FMT("mi_decoder_create: norm weights must be 8-byte aligned and hidden a multiple of 4");
+        delete d;
+        return nullptr;
+    }
 
     const int D = c.head_dim, kvd = c.n_kv_heads * D, qd = c.n_heads * D;
     const size_t cache = static_cast<size_t>(L) * c.max_pos * kvd * 2;
@@ -251,7 +316,6 @@ void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* 
               dev_alloc(d, &d->k, kvd * 2) && dev_alloc(d, &d->v, kvd * 2) && dev_alloc(d, &d->attn, qd * 2) &&
               dev_alloc(d, &d->proj, c.hidden * 2) && dev_alloc(d, &d->gate, c.inter * 2) &&
               dev_alloc(d, &d->up, c.inter * 2) && dev_alloc(d, &d->logits, static_cast<size_t>(c.vocab) * 2) &&
-              dev_alloc(d, &d->scores, static_cast<size_t>(c.n_heads) * c.max_pos * 2) &&
               dev_alloc(d, &d->st, sizeof(State));
     if (ok) {
         // rotary tables, QW/src/layers/attention.cpp:133-172: cos/sin(t * theta^(-2i/D)), both halves alike
@@ -330,52 +394,42 @@ int mi_decoder_step(void* dec, void* stream) {
     const int Hd = c.hidden, D = c.head_dim, qd = c.n_heads * D, kvd = c.n_kv_heads * D;
     const float scale = 1.0f / sqrtf(static_cast<float>(D));
     auto launched = [] { return MI_HIP_OK(hipGetLastError()); };
-    auto rmsnorm = [&](const uint16_t* x, const void* w, uint16_t* out) {
-        hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(64), 0, s, x, static_cast<const uint16_t*>(w), out, Hd, c.rms_eps);
-        return launched();
-    };
-    auto add = [&](const AddJobs& jobs, int nmax) {
-        hipLaunchKernelGGL(add_kernel, dim3((nmax + 255) / 256), dim3(256), 0, s, jobs);
+    // x (+= residual, if given), then out = rmsnorm(x) * w
+    auto rmsnorm = [&](uint16_t* x, const uint16_t* residual, const void* w, uint16_t* out) {
+        hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(64), 0, s, x, residual, static_cast<const uint16_t*>(w), out, Hd,
+                           c.rms_eps);
         return launched();
     };
     hipLaunchKernelGGL(embed_kernel, dim3(1), dim3(256), 0, s, static_cast<const uint16_t*>(d->embed), d->st, d->h, Hd, c.vocab);
     if (!launched()) return 0;
     for (int l = 0; l < c.n_layers; ++l) {
-        if (!rmsnorm(d->h, d->in_norm[l], d->xn)) return 0;
+        // the previous layer's down-projection residual is added here, ahead of this layer's first norm
+        if (!rmsnorm(d->h, l ? d->proj : nullptr, d->in_norm[l], d->xn)) return 0;
         const mi_linear_call qkv[3] = {{1, qd, Hd, d->xn, d->wq[l], d->q},
                                        {1, kvd, Hd, d->xn, d->wk[l], d->k},
                                        {1, kvd, Hd, d->xn, d->wv[l], d->v}};
         if (mi_linear_batch(stream, qkv, 3) != 3) return 0;
-        AddJobs bias{};
-        bias.j[0] = {d->q, static_cast<const uint16_t*>(d->bq[l]), qd};
-        bias.j[1] = {d->k, static_cast<const uint16_t*>(d->bk[l]), kvd};
-        bias.j[2] = {d->v, static_cast<const uint16_t*>(d->bv[l]), kvd};
-        bias.count = 3;
-        if (!add(bias, qd)) return 0;
         uint16_t* kc = d->kc + static_cast<size_t>(l) * c.max_pos * kvd;
         uint16_t* vc = d->vc + static_cast<size_t>(l) * c.max_pos * kvd;
         const int pairs = (c.n_heads + c.n_kv_heads) * D / 2;
-        hipLaunchKernelGGL(rope_kv_kernel, dim3((pairs + 255) / 256), dim3(256), 0, s, d->q, d->k, d->v, d->cosT, d->sinT,
-                           kc, vc, d->st, c.n_heads, c.n_kv_heads, D, c.max_pos);
+        hipLaunchKernelGGL(bias_rope_kv_kernel, dim3((pairs + 255) / 256), dim3(256), 0, s, d->q, d->k, d->v,
+                           static_cast<const uint16_t*>(d->bq[l]), static_cast<const uint16_t*>(d->bk[l]),
+                           static_cast<const uint16_t*>(d->bv[l]), d->cosT, d->sinT, kc, vc, d->st, c.n_heads,
+                           c.n_kv_heads, D, c.max_pos);
         if (!launched()) return 0;
         const int at = D > 64 ? D : 64;
-        hipLaunchKernelGGL(attention_kernel, dim3(c.n_heads), dim3(at), static_cast<size_t>(c.max_pos) * 4, s, d->q, kc, vc,
-                           d->scores, d->attn, d->st, c.n_heads, c.n_kv_heads, D, c.max_pos, scale);
+        hipLaunchKernelGGL(attention_kernel, dim3(c.n_heads), dim3(at), static_cast<size_t>(c.max_pos) * 6, s, d->q, kc, vc,
+                           d->attn, d->st, c.n_heads, c.n_kv_heads, D, c.max_pos, scale);
         if (!launched()) return 0;
         if (!mi_linear(stream, 1, Hd, qd, d->attn, d->wo[l], d->proj)) return 0;
-        AddJobs res{};
-        res.j[0] = {d->h, d->proj, Hd};
-        res.count = 1;
-        if (!add(res, Hd)) return 0;
-        if (!rmsnorm(d->h, d->post_norm[l], d->xn)) return 0;
+        if (!rmsnorm(d->h, d->proj, d->post_norm[l], d->xn)) return 0;          // h += o-projection, then the norm
         const mi_linear_call gu[2] = {{1, c.inter, Hd, d->xn, d->wgate[l], d->gate}, {1, c.inter, Hd, d->xn, d->wup[l], d->up}};
         if (mi_linear_batch(stream, gu, 2) != 2) return 0;
         hipLaunchKernelGGL(swiglu_kernel, dim3((c.inter + 255) / 256), dim3(256), 0, s, d->gate, d->up, c.inter);
         if (!launched()) return 0;
         if (!mi_linear(stream, 1, Hd, c.inter, d->gate, d->wdown[l], d->proj)) return 0;
-        if (!add(res, Hd)) return 0;
     }
-    if (!rmsnorm(d->h, d->final_norm, d->xn)) return 0;
+    if (!rmsnorm(d->h, d->proj, d->final_norm, d->xn)) return 0;                // the last residual add, then the final norm
     if (!mi_linear_argmax(stream, c.vocab, Hd, d->xn, d->lm_head, d->logits, 32,
                           reinterpret_cast<char*>(d->st) + offsetof(State, next)))
         return 0;
