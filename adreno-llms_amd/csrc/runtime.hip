@@ -330,7 +330,7 @@ void* mi_graph_end(void* stream) {
     if (!MI_HIP_OK(hipStreamEndCapture(as_stream(stream), &g)) || !g) return nullptr;
     hipGraphExec_t exec = nullptr;
     const bool ok = MI_HIP_OK(hipGraphInstantiate(&exec, g, nullptr, nullptr, 0));
-    hipGraphDestroy(g);
+    (void)hipGraphDestroy(g);      // the executable graph keeps what it needs
     return ok ? exec : nullptr;
 }
 
