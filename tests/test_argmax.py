@@ -136,3 +136,45 @@ def test_lm_head_then_argmax_on_device():
         mil.nnopt_unregister_weight(wb2)
     finally:
         mil.lib().mi_set_gemv_mode(1)
+
+
+@pytest.mark.gpu
+def test_stream_without_workspace_takes_the_one_launch_paths():
+    """A hipStream_t that mi_stream_create did not make has no workspace: the argmax runs as one
+    block and an int8 GEMM that would cut K into slices runs unsliced.  Same results."""
+    import ctypes
+    from helpers import synth_w, synth_x
+    assert mil.lib().mi_init(0) == 1
+    hip = ctypes.CDLL("libamdhip64.so")
+    foreign = ctypes.c_void_p()
+    assert hip.hipStreamCreate(ctypes.byref(foreign)) == 0
+    try:
+        own = mil.Queue()
+        x = np.random.default_rng(5).integers(-3, 4, 151936).astype(np.float16)     # thousands of ties
+        xb = mil.Buffer.from_host(x)
+        t_own, t_foreign = mil.Buffer.from_host(np.array([-1], np.int32)), mil.Buffer.from_host(np.array([-1], np.int32))
+        assert mil.argmax_f16(own, xb, x.size, t_own)
+        assert mil.lib().mi_argmax_f16(foreign, xb.ptr, x.size, 32, t_foreign.ptr)
+        own.finish()
+        assert hip.hipStreamSynchronize(foreign) == 0
+        want = O.argmax_f16(x)
+        assert int(t_own.read(np.int32, (1,))[0]) == want
+        assert int(t_foreign.read(np.int32, (1,))[0]) == want
+        # GEMM: 64 x 896 x 4864 is a shape the library slices along K when it has a workspace
+        M, N, K = 64, 896, 4864
+        W, X = synth_w(61, N, K), synth_x(62, M, K)
+        qw, s = mil.quantize_int8(W)
+        wb, sb, Xb = mil.Buffer.from_host(qw), mil.Buffer.from_host(s), mil.Buffer.from_host(X)
+        assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+        o_own, o_foreign = mil.Buffer(M * N * 2), mil.Buffer(M * N * 2)
+        assert mil.pytorch_linear(own, M, N, K, Xb, wb, o_own)
+        assert mil.lib().mi_linear(foreign, M, N, K, Xb.ptr, wb.ptr, o_foreign.ptr)
+        own.finish()
+        assert hip.hipStreamSynchronize(foreign) == 0
+        want = O.gemm_i8(X, qw, s.view(np.uint16)).view(np.float16)
+        from helpers import assert_tolerance
+        assert_tolerance(o_own.read(np.float16, (M, N)), want)
+        assert_tolerance(o_foreign.read(np.float16, (M, N)), want)
+        mil.nnopt_unregister_weight(wb)
+    finally:
+        hip.hipStreamDestroy(foreign)
