@@ -45,6 +45,18 @@ __device__ __forceinline__ void i8x4_to_h4(uint32_t v, uint32_t& lo, uint32_t& h
     hi = __builtin_bit_cast(uint32_t, __hsub2(__builtin_bit_cast(__half2, b), k));
 }
 
+// Byte B of v holds two Q4 values, low nibble first.  Returns them as a pair of fp16 times the
+// pair s2: the nibbles are placed into the mantissas of 1024 (unit 1) and of 64 (unit 1/16, which
+// is where a high nibble sits), 1032 and 72 are subtracted (exact), and the product with the
+// scale is rounded to fp16 once.
+template <int B>
+__device__ __forceinline__ uint32_t q4x2_to_h2(uint32_t v, __half2 s2) {
+    const uint32_t t = __builtin_amdgcn_perm(0u, v, 0x0C000C00u | (B << 16) | B);
+    const uint32_t h = (t & 0x00F0000Fu) | 0x54006400u;
+    const __half2 k = __builtin_bit_cast(__half2, 0xD480E408u);               // -1032, -72
+    return __builtin_bit_cast(uint32_t, __hmul2(__hadd2(__builtin_bit_cast(__half2, h), k), s2));
+}
+
 template <int BM, int BN, int WM, int WN, int KIND>
 __global__ __launch_bounds__(kThreads) void gemm_kernel(const uint16_t* __restrict__ X,
                                                         const uint8_t* __restrict__ W,
@@ -205,14 +217,25 @@ namespace wide {
 constexpr int kBN = 256;                    // rows of W per block
 // LDS stages (K = 64 each) for 32 * tm rows of x: as many as 160 KB hold, at most 8.  A stage is
 // requested stages - 2 stage times before it is needed, which is what covers the load latency.
-constexpr int stages_for(int tm) { return tm >= 4 ? 4 : tm == 3 ? 5 : tm == 2 ? 6 : 8; }
-constexpr int kWStage = kBN * 64;           // bytes of W (int8) per stage
+constexpr int stages_for(int kind, int tm) {
+    return kind == WK_Q4 ? (tm >= 5 ? 5 : tm == 4 ? 6 : tm == 3 ? 7 : 8) : (tm >= 4 ? 4 : tm == 3 ? 5 : tm == 2 ? 6 : 8);
+}
+// bytes of W per stage: int8 rows of 64 bytes; Q4 rows of 32 bytes of packed nibbles followed by
+// the 256 rows' two block scales (fp16) each
+constexpr int w_stage_bytes(int kind) { return kind == WK_Q4 ? kBN * 32 + kBN * 4 : kBN * 64; }
 typedef __attribute__((address_space(3))) uint8_t lds_u8;
 typedef __attribute__((address_space(1))) const uint8_t glb_u8;
 
 __device__ __forceinline__ void lds_fill16(const uint8_t* g, uint8_t* l) {
     __builtin_amdgcn_global_load_lds((glb_u8*)g, (lds_u8*)l, 16, 0, 0);   // address-space casts
 }
+__device__ __forceinline__ void lds_fill4(const uint8_t* g, uint8_t* l) {
+    __builtin_amdgcn_global_load_lds((glb_u8*)g, (lds_u8*)l, 4, 0, 0);
+}
+#define MI_LDS_READ8(dst, addr, imm) \
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(imm))
+#define MI_LDS_READ4(dst, addr, imm) \
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(imm))
 #define MI_LDS_READ16(dst, addr, imm) \
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(imm))
 #define MI_WAIT_LGKM(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n) : "memory")
@@ -242,24 +265,32 @@ __device__ __forceinline__ uint32_t pack_half2(float a, float b) {
 
 template <int TM>
 struct Frags {
-    u32x4 w[2];          // 16 int8 of two 32-row fragments of W, as read from LDS
+    u32x4 w[2];          // int8: 16 weights of two 32-row fragments of W, as read from LDS
+    uint2 w4[2];         // Q4: the same, 8 bytes
+    uint32_t ws[2];      // Q4: the two block scales of the stage, of the lane's row in either fragment
     uint32_t wf[2][2][4];  // the same as fp16: [fragment][MFMA of the pair][4 dwords = 8 halves]
+    uint32_t wg[2][2][4];  // Q4 in two terms: the second term
     u32x4 x[2][TM];      // [MFMA of the pair][32-row fragment of x], 8 halves each
 };
 
-template <int TM>
-__global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__ X,
+template <int TM, int KIND, int TERMS>
+__global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
                                                    const uint8_t* __restrict__ W,
                                                    const uint16_t* __restrict__ scale,
                                                    uint16_t* __restrict__ out, int M, int N, int K,
                                                    float* __restrict__ partial, int splits) {
     constexpr int BM = 32 * TM;
     constexpr int kXStage = BM * 128;                    // bytes of x (fp16) per stage
-    constexpr int kStage = kXStage + kWStage;
-    constexpr int kLoads = TM + 4;                       // global -> LDS loads per wavefront and stage
-    constexpr int kStages = stages_for(TM);
-    constexpr int kReads = 2 + 2 * TM;                   // LDS reads per set of fragments
-    constexpr int kMfmas = 4 * TM;                       // MFMAs per half stage (K = 32)
+    constexpr bool Q4 = KIND == WK_Q4;
+    constexpr int kWRow = Q4 ? 32 : 64;                  // bytes of one row of W per stage
+    constexpr int kWLoads = Q4 ? 3 : 4;                  // Q4: two loads of nibbles, one of scales
+    constexpr int kWReads = Q4 ? 4 : 2;                  // Q4: two fragments, two scale pairs
+    constexpr int kScaleAt = kXStage + kBN * 32;         // Q4: the scales of a stage, 4 bytes per row of W
+    constexpr int kStage = kXStage + w_stage_bytes(KIND);
+    constexpr int kLoads = TM + kWLoads;                 // global -> LDS loads per wavefront and stage
+    constexpr int kStages = stages_for(KIND, TM);
+    constexpr int kReads = kWReads + 2 * TM;             // LDS reads per set of fragments
+    constexpr int kMfmas = 4 * TM * TERMS;               // MFMAs per half stage (K = 32)
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     const int lane = threadIdx.x & 63;
@@ -292,6 +323,7 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
 
     // per-row scales of this lane's output columns, requested before anything else so that they
     // are in registers long before the epilogue: sc[u][rq] = 4 fp16 scales of columns nq .. nq + 3
+    // (Q4 has no per-row scale: the block scales travel with the weights)
     const bool cols4 = (N % 4) == 0 && reinterpret_cast<uintptr_t>(scale) % 8 == 0;
     uint2 sc[2][4];
     #pragma unroll
@@ -299,7 +331,9 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
         #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
             const int nq = n0 + 64 * w + 32 * u + 8 * rq + 4 * g;
-            if (cols4 && nq + 3 < N) {
+            if constexpr (Q4) {
+                sc[u][rq] = uint2{0u, 0u};
+            } else if (cols4 && nq + 3 < N) {
                 sc[u][rq] = *reinterpret_cast<const uint2*>(scale + nq);
             } else {
                 uint32_t h[4];
@@ -313,6 +347,9 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
     // --- fill side: lane i of load j writes LDS bytes [1024 j + 16 i, +16) of its region --------
     // x: load j covers rows 8j..8j+7 (128 bytes each, 8 chunks); slot p of row r holds chunk p ^ ((r >> 1) & 7)
     // W: load j covers rows 16j..16j+15 (64 bytes each, 4 chunks); slot p of row r holds chunk p ^ ((r >> 2) & 3)
+    // W, Q4: load j covers rows 32j..32j+31 (32 bytes each, 2 chunks); slot p of row r holds chunk
+    //        p ^ ((r >> 3) & 1); a third load of 4 bytes per lane brings the two block scales of
+    //        the wavefront's own 64 rows
     uint32_t xsrc[TM], wsrc[4];
     #pragma unroll
     for (int jj = 0; jj < TM; ++jj) {
@@ -321,13 +358,28 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
         const int m = m0 + r < M ? m0 + r : M - 1;
         xsrc[jj] = static_cast<uint32_t>(m) * K * 2u + c * 16u;
     }
-    #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-        const int r = 16 * (4 * w + jj) + (lane >> 2);
-        const int c = (lane & 3) ^ ((r >> 2) & 3);
+    if constexpr (Q4) {
+        #pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            const int r = 32 * (2 * w + jj) + (lane >> 1);
+            const int c = (lane & 1) ^ ((r >> 3) & 1);
+            const int n = n0 + r < N ? n0 + r : N - 1;
+            wsrc[jj] = static_cast<uint32_t>(n) * (K / 2) + c * 16u;
+        }
+        const int r = 64 * w + lane;
         const int n = n0 + r < N ? n0 + r : N - 1;
-        wsrc[jj] = static_cast<uint32_t>(n) * K + c * 16u;
+        wsrc[2] = static_cast<uint32_t>(n) * (K / 32) * 2u;
+        wsrc[3] = 0u;
+    } else {
+        #pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int r = 16 * (4 * w + jj) + (lane >> 2);
+            const int c = (lane & 3) ^ ((r >> 2) & 3);
+            const int n = n0 + r < N ? n0 + r : N - 1;
+            wsrc[jj] = static_cast<uint32_t>(n) * K + c * 16u;
+        }
     }
+    const uint8_t* Sb = reinterpret_cast<const uint8_t*>(scale);  // Q4: advanced like W below
     const uint8_t* Xb = reinterpret_cast<const uint8_t*>(X);     // both advanced to the block's first K-stage below
     // load j (0 .. kLoads - 1) of this wavefront for K-stage stage_k into LDS slot `slot`
     auto fill_one = [&](int stage_k, int slot, auto jc) {
@@ -335,8 +387,12 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
         uint8_t* xs = lds + slot * kStage;
         if constexpr (j < TM)
             lds_fill16(Xb + static_cast<size_t>(stage_k) * 128 + xsrc[j], xs + 1024 * (w + 4 * j));
-        else
+        else if constexpr (!Q4)
             lds_fill16(W + static_cast<size_t>(stage_k) * 64 + wsrc[j - TM], xs + kXStage + 1024 * (4 * w + (j - TM)));
+        else if constexpr (j - TM < 2)
+            lds_fill16(W + static_cast<size_t>(stage_k) * 32 + wsrc[j - TM], xs + kXStage + 1024 * (2 * w + (j - TM)));
+        else
+            lds_fill4(Sb + static_cast<size_t>(stage_k) * 4 + wsrc[2], xs + kScaleAt + 256 * w);
     };
     auto fill_stage = [&](int stage_k, int slot) {
         static_for<kLoads>([&](auto jc) { fill_one(stage_k, slot, jc); });
@@ -345,13 +401,15 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
     // --- read side -------------------------------------------------------------------------------
     // pair S (0, 1) of a stage, MFMA e (0, 1) of the pair: x chunk 4S + 2g + e, W chunk 2S + g
     const uint32_t xrow = lbase + li * 128u, xq = (2u * g) ^ ((li >> 1) & 7u);
-    const uint32_t wrow = lbase + kXStage + (64u * w + li) * 64u, wq = g ^ ((li >> 2) & 3u);
+    // Q4: bytes 16 S + 8 g .. + 7 of the row: chunk S, its lower or upper half
+    const uint32_t wrow = lbase + kXStage + (64u * w + li) * kWRow, wq = Q4 ? (li >> 3) & 1u : g ^ ((li >> 2) & 3u);
+    const uint32_t soff = lbase + kScaleAt + (64u * w + li) * 4u;
     uint32_t xoff[2][2], woff[2];
     #pragma unroll
     for (int S = 0; S < 2; ++S) {
         #pragma unroll
         for (int e = 0; e < 2; ++e) xoff[S][e] = xrow + (((4u * S + e) ^ xq) << 4);
-        woff[S] = wrow + (((2u * S) ^ wq) << 4);
+        woff[S] = Q4 ? wrow + ((S ^ wq) << 4) + 8u * g : wrow + (((2u * S) ^ wq) << 4);
     }
     // LDS read j (0 .. kReads - 1) of a set: the two W fragments first, then x for the first and
     // the second MFMA of the pair
@@ -359,17 +417,47 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
         constexpr int S = decltype(Sc)::value, j = decltype(jc)::value;
         if constexpr (j < 2) {
             const uint32_t a = woff[S] + slot_bytes;
-            MI_LDS_READ16(F.w[j], a, j * 32 * 64);
+            if constexpr (Q4) {
+                MI_LDS_READ8(F.w4[j], a, j * 32 * kWRow);
+            } else {
+                MI_LDS_READ16(F.w[j], a, j * 32 * kWRow);
+            }
+        } else if constexpr (j < kWReads) {
+            const uint32_t a = soff + slot_bytes;
+            MI_LDS_READ4(F.ws[j - 2], a, (j - 2) * 32 * 4);
         } else {
-            constexpr int e = (j - 2) / TM, t = (j - 2) % TM;
+            constexpr int e = (j - kWReads) / TM, t = (j - kWReads) % TM;
             const uint32_t a = xoff[S][e] + slot_bytes;
             MI_LDS_READ16(F.x[e][t], a, t * 4096);
         }
     };
     // conversion j (0 .. 7) of a set: dword j % 4 of W fragment j / 4 becomes four halves
-    auto convert_one = [&](Frags<TM>& F, auto jc) {
+    // Q4 (S = pair of the stage, which selects the block scale): bytes 2 (d % 2), 2 (d % 2) + 1 of
+    // dword d / 2 of fragment j / 4 become four halves, scaled
+    auto convert_one = [&](Frags<TM>& F, auto Sc, auto jc) {
         constexpr int j = decltype(jc)::value, u = j / 4, d = j % 4;
-        i8x4_to_h4(F.w[u][d], F.wf[u][d / 2][2 * (d % 2)], F.wf[u][d / 2][2 * (d % 2) + 1]);
+        if constexpr (Q4) {
+            constexpr int S = decltype(Sc)::value;
+            const uint32_t sb = __builtin_amdgcn_perm(0u, F.ws[u], S ? 0x03020302u : 0x01000100u);
+            const uint32_t v = d / 2 ? F.w4[u].y : F.w4[u].x;
+            if constexpr (TERMS == 2) {
+                // scale = hi + lo with 7 and 4 significant bits: q * hi and q * lo are exact in
+                // fp16 and add up to q * scale in the fp32 accumulator
+                const uint32_t hi = sb & 0xFFF0FFF0u;
+                const __half2 s2 = __builtin_bit_cast(__half2, hi);
+                const __half2 r2 = __hsub2(__builtin_bit_cast(__half2, sb), s2);
+                F.wf[u][d / 2][2 * (d % 2)] = q4x2_to_h2<2 * (d % 2)>(v, s2);
+                F.wf[u][d / 2][2 * (d % 2) + 1] = q4x2_to_h2<2 * (d % 2) + 1>(v, s2);
+                F.wg[u][d / 2][2 * (d % 2)] = q4x2_to_h2<2 * (d % 2)>(v, r2);
+                F.wg[u][d / 2][2 * (d % 2) + 1] = q4x2_to_h2<2 * (d % 2) + 1>(v, r2);
+            } else {
+                const __half2 s2 = __builtin_bit_cast(__half2, sb);
+                F.wf[u][d / 2][2 * (d % 2)] = q4x2_to_h2<2 * (d % 2)>(v, s2);
+                F.wf[u][d / 2][2 * (d % 2) + 1] = q4x2_to_h2<2 * (d % 2) + 1>(v, s2);
+            }
+        } else {
+            i8x4_to_h4(F.w[u][d], F.wf[u][d / 2][2 * (d % 2)], F.wf[u][d / 2][2 * (d % 2) + 1]);
+        }
     };
 
     floatx16 acc[2][TM];
@@ -382,8 +470,9 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
 
     // MFMA n (0 .. kMfmas - 1) of a half stage; consecutive n use different accumulators
     auto mfma_one = [&](const Frags<TM>& F, auto nc) {
-        constexpr int n = decltype(nc)::value, e = n / (2 * TM), u = (n / TM) % 2, t = n % TM;
-        const u32x4 wv = {F.wf[u][e][0], F.wf[u][e][1], F.wf[u][e][2], F.wf[u][e][3]};
+        constexpr int n = decltype(nc)::value, c = n / (2 * TM), e = c % 2, u = (n / TM) % 2, t = n % TM;
+        const u32x4 wv = c / 2 ? u32x4{F.wg[u][e][0], F.wg[u][e][1], F.wg[u][e][2], F.wg[u][e][3]}
+                               : u32x4{F.wf[u][e][0], F.wf[u][e][1], F.wf[u][e][2], F.wf[u][e][3]};
         acc[u][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, wv),
                                                           __builtin_bit_cast(half8, F.x[e][t]), acc[u][t], 0, 0, 0);
     };
@@ -413,10 +502,15 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
                 } else if constexpr (a == nF + kReads) {
                     // LDS returns in order: the two W reads are back.  The registers are operands
                     // of the wait so that the conversions that read them cannot be moved above it.
-                    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(Nx.w[0]), "+v"(Nx.w[1]) : "n"(kReads - 2) : "memory");
+                    if constexpr (Q4)
+                        asm volatile("s_waitcnt lgkmcnt(%4)"
+                                     : "+v"(Nx.w4[0]), "+v"(Nx.w4[1]), "+v"(Nx.ws[0]), "+v"(Nx.ws[1])
+                                     : "n"(kReads - kWReads) : "memory");
+                    else
+                        asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(Nx.w[0]), "+v"(Nx.w[1]) : "n"(kReads - kWReads) : "memory");
                     MI_SCHED_FENCE();
                 } else {
-                    convert_one(Nx, std::integral_constant<int, a - nF - kReads - 1>{});
+                    convert_one(Nx, NSc, std::integral_constant<int, a - nF - kReads - 1>{});
                 }
             });
             MI_SCHED_FENCE();
@@ -444,7 +538,8 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
     const int k_first = static_cast<int>(static_cast<long>(K / 64) * split / splits);
     const int nk = static_cast<int>(static_cast<long>(K / 64) * (split + 1) / splits) - k_first;
     Xb += static_cast<size_t>(k_first) * 128;
-    W += static_cast<size_t>(k_first) * 64;
+    W += static_cast<size_t>(k_first) * kWRow;
+    Sb += static_cast<size_t>(k_first) * 4;
     Frags<TM> FA, FB;
     #pragma unroll
     for (int st = 0; st < kStages - 1; ++st)
@@ -453,9 +548,12 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
     __builtin_amdgcn_s_barrier();
     MI_SCHED_FENCE();
     static_for<kReads>([&](auto jc) { read_one(FA, 0u, std::integral_constant<int, 0>{}, jc); });
-    MI_WAIT_LGKM(0);
+    if constexpr (Q4)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(FA.w4[0]), "+v"(FA.w4[1]), "+v"(FA.ws[0]), "+v"(FA.ws[1]) : : "memory");
+    else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(FA.w[0]), "+v"(FA.w[1]) : : "memory");
     MI_SCHED_FENCE();
-    static_for<8>([&](auto jc) { convert_one(FA, jc); });
+    static_for<8>([&](auto jc) { convert_one(FA, std::integral_constant<int, 0>{}, jc); });
 
     // Stage i lives in slot i % kStages.  In the middle of stage i every wavefront waits for its
     // own fills of stage i + 1 and meets the others at the barrier; behind it stage i + 1 is
@@ -526,11 +624,13 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
     for (int u = 0; u < 2; ++u) {
         #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
-            float s4[4];
-            s4[0] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].x & 0xFFFFu)));
-            s4[1] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].x >> 16)));
-            s4[2] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].y & 0xFFFFu)));
-            s4[3] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].y >> 16)));
+            float s4[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+            if constexpr (!Q4) {
+                s4[0] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].x & 0xFFFFu)));
+                s4[1] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].x >> 16)));
+                s4[2] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].y & 0xFFFFu)));
+                s4[3] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].y >> 16)));
+            }
             #pragma unroll
             for (int t = 0; t < TM; ++t) {
                 const uint32_t lo = pack_half2(acc[u][t][4 * rq] * s4[0], acc[u][t][4 * rq + 1] * s4[1]);
@@ -559,8 +659,9 @@ __global__ __launch_bounds__(256) void gemm_i8_wide(const uint16_t* __restrict__
     }
 }
 
-// out[m][n] = fp16((sum over slices of partial[slice][m][n]) * scale[n]); slices are added in
-// index order, so the result does not depend on how the blocks were scheduled.
+// out[m][n] = fp16((sum over slices of partial[slice][m][n]) * scale[n]) (no factor when scale is
+// null); slices are added in index order, so the result does not depend on how the blocks were
+// scheduled.
 __global__ __launch_bounds__(256) void reduce_partials(const float* __restrict__ partial, int splits,
                                                        const uint16_t* __restrict__ scale,
                                                        uint16_t* __restrict__ out, long MN, int N) {
@@ -574,23 +675,26 @@ __global__ __launch_bounds__(256) void reduce_partials(const float* __restrict__
             a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
         }
         const int n = static_cast<int>(i4 % N);
-        const float s0 = __half2float(__ushort_as_half(scale[n])), s1 = __half2float(__ushort_as_half(scale[n + 1]));
-        const float s2 = __half2float(__ushort_as_half(scale[n + 2])), s3 = __half2float(__ushort_as_half(scale[n + 3]));
+        float s0 = 1.0f, s1 = 1.0f, s2 = 1.0f, s3 = 1.0f;
+        if (scale) {
+            s0 = __half2float(__ushort_as_half(scale[n])), s1 = __half2float(__ushort_as_half(scale[n + 1]));
+            s2 = __half2float(__ushort_as_half(scale[n + 2])), s3 = __half2float(__ushort_as_half(scale[n + 3]));
+        }
         *reinterpret_cast<uint2*>(out + i4) = uint2{pack_half2(a.x * s0, a.y * s1), pack_half2(a.z * s2, a.w * s3)};
     } else {
         for (int e = 0; e < 4 && i4 + e < MN; ++e) {
             float a = partial[i4 + e];
             for (int z = 1; z < splits; ++z) a += partial[z * MN + i4 + e];
-            out[i4 + e] = to_half_bits(a * __half2float(__ushort_as_half(scale[(i4 + e) % N])));
+            out[i4 + e] = to_half_bits(scale ? a * __half2float(__ushort_as_half(scale[(i4 + e) % N])) : a);
         }
     }
 }
 
-template <int TM>
+template <int TM, int KIND, int TERMS>
 bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out,
             float* partial, int splits) {
-    constexpr size_t lds_bytes = static_cast<size_t>(stages_for(TM)) * (32 * TM * 128 + kWStage);
-    auto* kern = gemm_i8_wide<TM>;
+    constexpr size_t lds_bytes = static_cast<size_t>(stages_for(KIND, TM)) * (32 * TM * 128 + w_stage_bytes(KIND));
+    auto* kern = gemm_wide<TM, KIND, TERMS>;
     static bool raised = false;
     if (lds_bytes > 65536 && !raised) {
         if (!MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -606,7 +710,8 @@ bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, co
     if (splits > 1) {
         const long MN = static_cast<long>(M) * N;
         hipLaunchKernelGGL(reduce_partials, dim3(static_cast<unsigned>((MN / 4 + 256) / 256)), dim3(256), 0, s,
-                           partial, splits, static_cast<const uint16_t*>(scale), static_cast<uint16_t*>(out), MN, N);
+                           partial, splits, KIND == WK_Q4 ? nullptr : static_cast<const uint16_t*>(scale),
+                           static_cast<uint16_t*>(out), MN, N);
         if (!MI_HIP_OK(hipGetLastError())) return false;
     }
     return true;
@@ -614,13 +719,16 @@ bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, co
 
 // Estimated time (us) of the wide kernel with 32 * tm rows of x per block and K cut into
 // `splits` slices.  Fitted to measurements on MI355X: a block takes about 2.6 + 0.5 tm us of
-// prologue and epilogue plus, per K-stage of 64, 0.27 + 0.10 tm us; a fully occupied chip runs
-// the same cycles about 1.56 times slower (clock under load, shared L2 and fabric) than a nearly
-// empty one.  Slices cost a second launch and the partial sums' trip through memory.
-inline double estimate_us(int tm, int splits, int M, int N, int K, int cus) {
+// prologue and epilogue plus, per K-stage of 64, 0.27 + 0.10 tm us for int8 weights, 0.56 + 0.10 tm
+// for Q4 weights rounded to fp16 once and 0.49 + 0.22 tm for Q4 weights in two terms; a fully
+// occupied chip runs the same cycles about 1.56 times slower (clock under load, shared L2 and
+// fabric) than a nearly empty one.  Slices cost a second launch and the partial sums' trip
+// through memory.
+inline double estimate_us(int kind, int terms, int tm, int splits, int M, int N, int K, int cus) {
     const long blocks = static_cast<long>((M + 32 * tm - 1) / (32 * tm)) * ((N + kBN - 1) / kBN) * splits;
     const int stages = (K / 64 + splits - 1) / splits;
-    const double block_us = 2.6 + 0.5 * tm + stages * (0.27 + 0.10 * tm);
+    const double stage_us = kind == WK_Q4 ? (terms == 2 ? 0.49 + 0.22 * tm : 0.56 + 0.10 * tm) : 0.27 + 0.10 * tm;
+    const double block_us = 2.6 + 0.5 * tm + stages * stage_us;
     const long full = blocks / cus, rem = blocks % cus;
     double t = full * 1.56 * block_us + (rem ? (1.0 + 0.56 * rem / cus) * block_us : 0.0);
     if (splits > 1) t += 2.5 + 2.0 * splits * M * static_cast<double>(N) * 4 / 4.0e6;   // ~4 TB/s there and back
@@ -629,29 +737,30 @@ inline double estimate_us(int tm, int splits, int M, int N, int K, int cus) {
 
 // Rows of x per block (in units of 32) and slices of K with the smallest estimated time; slices
 // only as far as their fp32 partial sums fit the workspace.
-inline void pick_shape(int M, int N, int K, int cus, size_t workspace_bytes, int* tm_out, int* splits_out,
-                       double* best_us) {
+inline void pick_shape(int kind, int terms, int M, int N, int K, int cus, size_t workspace_bytes, int* tm_out,
+                       int* splits_out, double* best_us) {
     static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24};
     double best_t = 1e30;
     for (int tm = 1; tm <= 5; ++tm) {
         for (int sp : kSplits) {
             if (sp > 1 && (K / 64 < 2 * sp || static_cast<double>(sp) * M * N * 4 > static_cast<double>(workspace_bytes)))
                 continue;
-            const double t = estimate_us(tm, sp, M, N, K, cus);
+            const double t = estimate_us(kind, terms, tm, sp, M, N, K, cus);
             if (t < best_t) { best_t = t; *tm_out = tm; *splits_out = sp; }
         }
     }
     if (best_us) *best_us = best_t;
 }
 
-inline bool launch_any(int tm, hipStream_t s, int M, int N, int K, const void* x, const void* W,
-                       const void* scale, void* out, float* partial, int splits) {
+template <int KIND, int TERMS>
+bool launch_any(int tm, hipStream_t s, int M, int N, int K, const void* x, const void* W,
+                const void* scale, void* out, float* partial, int splits) {
     switch (tm) {
-        case 1: return launch<1>(s, M, N, K, x, W, scale, out, partial, splits);
-        case 2: return launch<2>(s, M, N, K, x, W, scale, out, partial, splits);
-        case 3: return launch<3>(s, M, N, K, x, W, scale, out, partial, splits);
-        case 4: return launch<4>(s, M, N, K, x, W, scale, out, partial, splits);
-        default: return launch<5>(s, M, N, K, x, W, scale, out, partial, splits);
+        case 1: return launch<1, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, splits);
+        case 2: return launch<2, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, splits);
+        case 3: return launch<3, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, splits);
+        case 4: return launch<4, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, splits);
+        default: return launch<5, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, splits);
     }
 }
 
@@ -695,7 +804,7 @@ inline long tiles(int M, int N, int bm, int bn) {
 }  // namespace
 
 bool gemm_supported(WeightKind kind, int M, int N, int K) {
-    return (kind == WK_I8 || kind == WK_F16) && M >= 16 && N >= 1 && K >= kKT && K % kKT == 0;
+    return (kind == WK_I8 || kind == WK_F16 || kind == WK_Q4) && M >= 16 && N >= 1 && K >= kKT && K % kKT == 0;
 }
 
 bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x, const void* W,
@@ -705,22 +814,40 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
         return false;
     }
     if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(W) % 16 ||
-        (kind == WK_I8 && !scale)) {
-        MI_ERROR_FMT("gemm: x and W must be 16-byte aligned, int8 needs a scale");
+        (kind != WK_F16 && !scale) || (kind == WK_Q4 && reinterpret_cast<uintptr_t>(scale) % 4)) {
+        MI_ERROR_FMT("gemm: x and W must be 16-byte aligned; int8 and Q4 need a scale, Q4 a 4-byte aligned one");
         return false;
     }
-    const int mode = gemm_mode();
+    const int mode = gemm_mode() == 4 && kind != WK_Q4 ? 0 : gemm_mode();   // mode 4 only concerns Q4 weights
     const int cus = device_info().cus;
     // int8: the wide kernel where its estimated time beats that of the 64 x 64 tiles, which are
     // bound either by one tile's serial K loop (about 0.4 us per K-tile, up to 1.3 times that as
     // the chip fills) or by throughput (1.2 to 1.55 ns per tile and K-tile); fitted to measurements
-    const bool wide_fits = kind == WK_I8 && static_cast<double>(M) * K * 2 < 4294967296.0 &&
+    const bool wide_fits = kind != WK_F16 && static_cast<double>(M) * K * 2 < 4294967296.0 &&
                            static_cast<double>(N) * K < 4294967296.0;   // 32-bit byte offsets
+    if (kind == WK_Q4) {
+        // Q4 weights have the wide kernel only; modes 3 and 11..15 pin it to one slice of K.
+        // Mode 4 feeds every weight as the single fp16 number nearest to q * scale (half the
+        // MFMAs, an error of up to 2^-12 sum |w x|); all other modes feed q * scale exactly, as
+        // two fp16 terms.
+        if (!wide_fits || mode == 2) {
+            MI_ERROR_FMT("gemm: Q4 weights take the wide kernel only (mode %d, M=%d N=%d K=%d)", mode, M, N, K);
+            return false;
+        }
+        const int terms = mode == 4 ? 1 : 2;
+        const bool may_slice = (mode == 0 || mode == 4) && workspace;
+        int tm = 1, splits = 1;
+        wide::pick_shape(WK_Q4, terms, M, N, K, cus, may_slice ? workspace_bytes : 0, &tm, &splits, nullptr);
+        if (mode >= 11 && mode <= 15) tm = mode - 10;
+        if (terms == 1)
+            return wide::launch_any<WK_Q4, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), splits);
+        return wide::launch_any<WK_Q4, 2>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), splits);
+    }
     if (wide_fits && (mode == 0 || mode == 3 || (mode >= 11 && mode <= 15))) {
         double wide_us = 0.0;
         int tm = 1, splits = 1;
         // modes 3 and 11..15 pin the plain kernel; slices of K are the library's own choice (mode 0)
-        wide::pick_shape(M, N, K, cus, mode == 0 && workspace ? workspace_bytes : 0, &tm, &splits, &wide_us);
+        wide::pick_shape(WK_I8, 1, M, N, K, cus, mode == 0 && workspace ? workspace_bytes : 0, &tm, &splits, &wide_us);
         const int nk = K / kKT;
         const long t64 = tiles(M, N, 64, 64);
         const double serial = (0.9 + nk * 0.4) * (1.0 + 0.3 * (t64 < 128 ? t64 / 128.0 : 1.0));
@@ -728,7 +855,7 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
         const double tiled_us = serial > bulk ? serial : bulk;
         if (mode >= 11) tm = mode - 10;
         if (mode != 0 || wide_us < tiled_us)
-            return wide::launch_any(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), splits);
+            return wide::launch_any<WK_I8, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), splits);
     } else if (mode == 3 || mode >= 11) {
         MI_ERROR_FMT("gemm: mode %d asks for the wide int8 kernel, which does not take kind=%d M=%d N=%d K=%d",
                      mode, static_cast<int>(kind), M, N, K);

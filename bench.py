@@ -278,6 +278,27 @@ def main():
                     "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                     "frac_hbm": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
             mil.nnopt_unregister_weight(wb)
+        # the same contraction with Q4 weights: exact two-term feed (default) and single rounding (mode 4)
+        N, K = INTER, H
+        ph, sh = mil.quantize_q4(mil.synth_normal_f16(77, 0.02, (N, K)))
+        wb, sb = mil.Buffer.from_host(ph), mil.Buffer.from_host(sh)
+        assert mil.nnopt_register_q4_weight(wb, sb, N, K)
+        for M in (16, 2048):
+            xb = mil.Buffer.from_host(mil.synth_normal_f16(78, 1.0, (M, K)))
+            ob = mil.Buffer(M * N * 2)
+            arr = mil.make_calls([(M, N, K, xb, wb, ob)] * 20)
+            for mode, tag in ((0, "q4"), (4, "q4_single_rounding")):
+                mil.lib().mi_set_gemm_mode(mode)
+                try:
+                    mil.linear_batch(queue, arr)
+                    ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 5) / 20
+                finally:
+                    mil.lib().mi_set_gemm_mode(0)
+                flop = 2.0 * M * N * K
+                detail[f"c5_{tag}_gemm_M{M}_N{N}_K{K}"] = {
+                    "us": round(ms * 1e3, 2), "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 1),
+                    "frac_mfma_fp16_peak": round(flop / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)}
+        mil.nnopt_unregister_weight(wb)
 
     # ---- CPU baseline: the oracle on a bounded sample of the same sweep -------------------
     cpu = None

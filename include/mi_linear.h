@@ -140,9 +140,14 @@ int   mi_graph_destroy(void* graph);
  * dequant for M >= 16 and batched GEMV below; 1 = always the batched GEMV, whose rows
  * are bit-identical to M = 1 calls (the reference's prefill loop, LF/src/model.cpp:243-250);
  * 2, 3 and 11..15 = as 0 with the kernel choice pinned (tests and tuning: results stay within
- * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel, 3 = the wide int8
- * kernel, 10 + t (t = 1..5) = the wide int8 kernel with 32 t rows of x per block; 3 and 10 + t
- * fail for weights that are not int8. */
+ * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel (int8 and fp16
+ * weights), 3 = the wide kernel, 10 + t (t = 1..5) = the wide kernel with 32 t rows of x per
+ * block; 3 and 10 + t take int8 and Q4 weights and fail for fp16 weights.
+ * Q4 weights: a weight q * scale (4 and 11 significant bits) is not an fp16 number in general.
+ * Every mode but 4 feeds it to the matrix cores exactly, as two fp16 terms q * hi + q * lo with
+ * scale = hi + lo, and stays within one fp16 step of the batched GEMV.  Mode 4 = as 0, but each
+ * Q4 weight is rounded to the nearest fp16 number first: half the matrix work (about 1.5 times
+ * faster), at an error of up to 2^-12 * sum_k |w x| on top; it changes nothing for other weights. */
 void mi_set_gemm_mode(int mode);
 
 /* Selects the M = 1 arithmetic.  0 = every GEMV evaluates the reference kernels' sum in the

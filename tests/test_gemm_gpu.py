@@ -35,12 +35,15 @@ def _ulp_apart(a_u16, b_u16):
 
 def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0):
     """tile is the mi_set_gemm_mode value: 0 = the library's own choice, 1 = rows of GEMV,
-    2 = the 64 x 64 MFMA kernel, 3 = the wide int8 kernel with its own choice of rows of x per
-    block, 11..15 = the wide kernel with 32, 64, .. 160 rows of x per block (int8 only)."""
+    2 = the 64 x 64 MFMA kernel, 3 = the wide kernel with its own choice of rows of x per
+    block, 4 = Q4 weights rounded to fp16 once, 11..15 = the wide kernel with 32, 64, .. 160 rows
+    of x per block (int8 and Q4)."""
     xb, wb = mil.Buffer.from_host(X), mil.Buffer.from_host(W_host)
     sb = mil.Buffer.from_host(scale_host) if scale_host is not None else None
     if kind == "i8":
         assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+    elif kind == "q4":
+        assert mil.nnopt_register_q4_weight(wb, sb, N, K)
     pad = 128
     guard = np.full(M * N + 2 * pad, 0x7BCD, np.uint16)
     ob = mil.Buffer.from_host(guard)
@@ -135,6 +138,139 @@ def test_gemm_repeats_identically(queue, tile):
     for i, ob in enumerate(outs[1:]):
         assert np.array_equal(ob.read(np.uint16, (M, N)), first), f"launch {i + 1} differs from launch 0"
     mil.nnopt_unregister_weight(wb)
+
+
+def _q4_values(p):
+    """[N, K/2] packed bytes -> [N, K] integers in -8..7 (low nibble first)."""
+    v = np.empty((p.shape[0], p.shape[1] * 2), np.int32)
+    v[:, 0::2] = p & 15
+    v[:, 1::2] = p >> 4
+    return v - 8
+
+
+@pytest.mark.parametrize("tile", [0, 3, 11, 12, 13, 14, 15])
+@pytest.mark.parametrize("M", [16, 64, 100, 512])
+@pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (200, 128), (130, 576), (131, 64)])
+def test_q4_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
+    """Q4 weights on the matrix cores.  A weight q * s (4 and 11 significant bits) is not an fp16
+    number in general, so the kernel feeds it as two: q * hi + q * lo with s = hi + lo, hi the 7
+    leading bits of s; both products are exact in fp16 and meet in the fp32 accumulator.  The bar
+    is then the same as for int8: at most one fp16 step from the rows of GEMV."""
+    print(f"q4 gemm M={M} N={N} K={K} tile mode {tile}", flush=True)
+    W, X = synth_w(1700 + N, N, K), synth_x(1800 + M, M, K)
+    p, s = mil.quantize_q4(W)
+    got = _gemm(queue, M, N, K, X, p, s, "q4", tile)
+    want = O.gemm_q4(X, p, s.view(np.uint16))
+    assert_tolerance(got.view(np.float16), want.view(np.float16))
+    d = _ulp_apart(got, want)
+    assert d.max() <= 1, f"max {d.max()} fp16 steps apart"
+    assert np.mean(got == want) > 0.99
+    # and from the exact value of the sum, rounded once
+    wt = _q4_values(p).astype(np.float64) * np.repeat(s.astype(np.float64), 32, axis=1)
+    exact = X.astype(np.float64) @ wt.T
+    assert _ulp_apart(got, exact.astype(np.float16).view(np.uint16)).max() <= 1
+
+
+@pytest.mark.parametrize("M", [16, 100, 512])
+@pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (130, 576)])
+def test_q4_gemm_single_rounding_mode_within_its_bound(queue, M, N, K):
+    """Mode 4: a weight enters as the one fp16 number nearest to q * scale.  Checked against the
+    a-priori bound of that rounding on top of one fp16 step, 2^-12 sum |w x|, and to one fp16
+    step against the exact sum over the rounded weights."""
+    W, X = synth_w(1700 + N, N, K), synth_x(1800 + M, M, K)
+    p, s = mil.quantize_q4(W)
+    got = _gemm(queue, M, N, K, X, p, s, "q4", 4)
+    want = O.gemm_q4(X, p, s.view(np.uint16))
+    wf = (_q4_values(p).astype(np.float32) * np.repeat(s.astype(np.float32), 32, axis=1)).astype(np.float16)
+    g, w = got.view(np.float16).astype(np.float64), want.view(np.float16).astype(np.float64)
+    bound = (2.0 ** -12 + 2.0 ** -20) * (np.abs(X).astype(np.float64) @ np.abs(wf).astype(np.float64).T) \
+        + np.spacing(np.abs(want.view(np.float16))).astype(np.float64)
+    assert np.all(np.abs(g - w) <= bound), f"worst excess {(np.abs(g - w) - bound).max()}"
+    cos = np.dot(g.ravel(), w.ravel()) / (np.linalg.norm(g) * np.linalg.norm(w))
+    assert cos >= 0.9999
+    exact = X.astype(np.float64) @ wf.astype(np.float64).T
+    assert _ulp_apart(got, exact.astype(np.float16).view(np.uint16)).max() <= 1
+
+
+def test_q4_gemm_tiny_scales_keep_fp16_subnormals(queue):
+    """Weights around 1e-4: the block scales and most products q * scale are fp16 subnormals.
+    They must enter the sums at full value (nothing flushed to zero on the way to the matrix cores)."""
+    M, N, K = 64, 512, 896
+    W = (synth_w(1960, N, K).astype(np.float32) * np.float32(0.004)).astype(np.float16)
+    X = (synth_x(1961, M, K).astype(np.float32) * np.float32(30.0)).astype(np.float16)
+    p, s = mil.quantize_q4(W)
+    assert np.mean(s.astype(np.float32) < 6.1e-5) > 0.9, "scales meant to be subnormal"
+    got = _gemm(queue, M, N, K, X, p, s, "q4")
+    want = O.gemm_q4(X, p, s.view(np.uint16))
+    assert np.abs(want.view(np.float16).astype(np.float32)).mean() > 0.01
+    assert _ulp_apart(got, want).max() <= 1
+
+
+@pytest.mark.parametrize("tile", [3, 4, 11, 13, 15])
+def test_q4_gemm_exact_on_integer_data(queue, tile):
+    # power-of-two scales and small integer x: every product and partial sum is exact
+    rng = np.random.default_rng(5)
+    M, N, K = 96, 192, 256
+    p = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
+    s = (2.0 ** rng.integers(-10, -6, (N, K // 32))).astype(np.float16)
+    X = rng.integers(-3, 4, (M, K)).astype(np.float16)
+    got = _gemm(queue, M, N, K, X, p, s, "q4", tile)
+    wf = _q4_values(p).astype(np.float64) * np.repeat(s.astype(np.float64), 32, axis=1)
+    want = (X.astype(np.float64) @ wf.T).astype(np.float16)
+    assert np.array_equal(got.view(np.float16), want)
+    assert np.array_equal(got, O.gemm_q4(X, p, s.view(np.uint16)))
+
+
+@pytest.mark.parametrize("tile", [3, 4, 12, 14, 15])
+def test_q4_gemm_unit_rows_pick_weight_columns(queue, tile):
+    # x rows are unit vectors: out[i, :] must be fp16(q * s) of column k_i (nibble order, block of the scale)
+    M, N, K = 64, 320, 896
+    p, s = mil.quantize_q4(synth_w(1910, N, K))
+    ks = (np.arange(M) * 37 + 5) % K
+    X = np.zeros((M, K), np.float16)
+    X[np.arange(M), ks] = 1.0
+    got = _gemm(queue, M, N, K, X, p, s, "q4", tile).view(np.float16)
+    want = (_q4_values(p)[:, ks].T.astype(np.float32) * s.astype(np.float32)[:, ks // 32].T).astype(np.float16)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("tile", [4, 11, 12, 13, 14, 15])
+def test_q4_gemm_repeats_identically(queue, tile):
+    M, N, K = 100, 1000, 1024
+    print(f"q4 repeat tile mode {tile}", flush=True)
+    W, X = synth_w(1940, N, K), synth_x(1941, M, K)
+    p, s = mil.quantize_q4(W)
+    want = O.gemm_q4(X, p, s.view(np.uint16))
+    xb, wb, sb = mil.Buffer.from_host(X), mil.Buffer.from_host(p), mil.Buffer.from_host(s)
+    assert mil.nnopt_register_q4_weight(wb, sb, N, K)
+    outs = [mil.Buffer(M * N * 2) for _ in range(25)]
+    mil.lib().mi_set_gemm_mode(tile)
+    try:
+        for ob in outs:
+            assert mil.pytorch_linear(queue, M, N, K, xb, wb, ob)
+        queue.finish()
+    finally:
+        mil.lib().mi_set_gemm_mode(0)
+    first = outs[0].read(np.uint16, (M, N))
+    assert_tolerance(first.view(np.float16), want.view(np.float16))
+    for i, ob in enumerate(outs[1:]):
+        assert np.array_equal(ob.read(np.uint16, (M, N)), first), f"launch {i + 1} differs from launch 0"
+    mil.nnopt_unregister_weight(wb)
+
+
+def test_q4_prefill_size_rows_sampled(queue):
+    M, N, K = 2048, 4864, 896
+    W, X = synth_w(1920, N, K), synth_x(1921, M, K)
+    p, s = mil.quantize_q4(W)
+    got = _gemm(queue, M, N, K, X, p, s, "q4")
+    for r in [0, 1, 31, 32, 159, 160, 1000, 1023, 1024, 2046, 2047]:
+        want = O.gemv_q4(X[r], p, s.view(np.uint16))
+        assert _ulp_apart(got[r], want).max() <= 1, f"row {r}"
+    X2 = X.copy()
+    X2[5] = X[5] * np.float16(2.0)
+    got2 = _gemm(queue, M, N, K, X2, p, s, "q4")
+    assert np.array_equal(got2[5].view(np.float16), got[5].view(np.float16) * np.float16(2.0))
+    assert np.array_equal(got2[6], got[6])
 
 
 def test_prefill_size_rows_sampled(queue):
