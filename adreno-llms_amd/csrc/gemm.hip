@@ -218,11 +218,15 @@ constexpr int kBN = 256;                    // rows of W per block
 // LDS stages (K = 64 each) for 32 * tm rows of x: as many as 160 KB hold, at most 8.  A stage is
 // requested stages - 2 stage times before it is needed, which is what covers the load latency.
 constexpr int stages_for(int kind, int tm) {
-    return kind == WK_Q4 ? (tm >= 5 ? 5 : tm == 4 ? 6 : tm == 3 ? 7 : 8) : (tm >= 4 ? 4 : tm == 3 ? 5 : tm == 2 ? 6 : 8);
+    return kind == WK_Q4 ? (tm >= 5 ? 5 : tm == 4 ? 6 : tm == 3 ? 7 : 8)
+         : kind == WK_F16 ? (tm >= 3 ? 3 : 4)
+                          : (tm >= 4 ? 4 : tm == 3 ? 5 : tm == 2 ? 6 : 8);
 }
-// bytes of W per stage: int8 rows of 64 bytes; Q4 rows of 32 bytes of packed nibbles followed by
-// the 256 rows' two block scales (fp16) each
-constexpr int w_stage_bytes(int kind) { return kind == WK_Q4 ? kBN * 32 + kBN * 4 : kBN * 64; }
+// bytes of W per stage: int8 rows of 64 bytes; fp16 rows of 128 bytes; Q4 rows of 32 bytes of
+// packed nibbles followed by the 256 rows' two block scales (fp16) each
+constexpr int w_stage_bytes(int kind) {
+    return kind == WK_Q4 ? kBN * 32 + kBN * 4 : kind == WK_F16 ? kBN * 128 : kBN * 64;
+}
 typedef __attribute__((address_space(3))) uint8_t lds_u8;
 typedef __attribute__((address_space(1))) const uint8_t glb_u8;
 
@@ -270,6 +274,7 @@ struct Frags {
     uint32_t ws[2];      // Q4: the two block scales of the stage, of the lane's row in either fragment
     uint32_t wf[2][2][4];  // the same as fp16: [fragment][MFMA of the pair][4 dwords = 8 halves]
     uint32_t wg[2][2][4];  // Q4 in two terms: the second term
+    u32x4 wh[2][2];        // fp16 weights: read from LDS as they are used
     u32x4 x[2][TM];      // [MFMA of the pair][32-row fragment of x], 8 halves each
 };
 
@@ -281,10 +286,11 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
                                                    float* __restrict__ partial, int splits) {
     constexpr int BM = 32 * TM;
     constexpr int kXStage = BM * 128;                    // bytes of x (fp16) per stage
-    constexpr bool Q4 = KIND == WK_Q4;
-    constexpr int kWRow = Q4 ? 32 : 64;                  // bytes of one row of W per stage
-    constexpr int kWLoads = Q4 ? 3 : 4;                  // Q4: two loads of nibbles, one of scales
-    constexpr int kWReads = Q4 ? 4 : 2;                  // Q4: two fragments, two scale pairs
+    constexpr bool Q4 = KIND == WK_Q4, F16 = KIND == WK_F16;
+    constexpr int kWRow = Q4 ? 32 : F16 ? 128 : 64;      // bytes of one row of W per stage
+    constexpr int kWLoads = Q4 ? 3 : F16 ? 8 : 4;        // Q4: two loads of nibbles, one of scales
+    constexpr int kWReads = Q4 || F16 ? 4 : 2;           // Q4: two fragments, two scale pairs; fp16: two fragments for two MFMAs
+    constexpr int kConv = F16 ? 0 : 8;                   // conversions per set of fragments
     constexpr int kScaleAt = kXStage + kBN * 32;         // Q4: the scales of a stage, 4 bytes per row of W
     constexpr int kStage = kXStage + w_stage_bytes(KIND);
     constexpr int kLoads = TM + kWLoads;                 // global -> LDS loads per wavefront and stage
@@ -331,7 +337,7 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
         #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
             const int nq = n0 + 64 * w + 32 * u + 8 * rq + 4 * g;
-            if constexpr (Q4) {
+            if constexpr (Q4 || F16) {
                 sc[u][rq] = uint2{0u, 0u};
             } else if (cols4 && nq + 3 < N) {
                 sc[u][rq] = *reinterpret_cast<const uint2*>(scale + nq);
@@ -350,7 +356,8 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
     // W, Q4: load j covers rows 32j..32j+31 (32 bytes each, 2 chunks); slot p of row r holds chunk
     //        p ^ ((r >> 3) & 1); a third load of 4 bytes per lane brings the two block scales of
     //        the wavefront's own 64 rows
-    uint32_t xsrc[TM], wsrc[4];
+    // W, fp16: as x, load j covers rows 8j..8j+7, eight loads for the wavefront's own 64 rows
+    uint32_t xsrc[TM], wsrc[F16 ? 8 : 4];
     #pragma unroll
     for (int jj = 0; jj < TM; ++jj) {
         const int r = 8 * (w + 4 * jj) + (lane >> 3);
@@ -370,6 +377,14 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
         const int n = n0 + r < N ? n0 + r : N - 1;
         wsrc[2] = static_cast<uint32_t>(n) * (K / 32) * 2u;
         wsrc[3] = 0u;
+    } else if constexpr (F16) {
+        #pragma unroll
+        for (int jj = 0; jj < 8; ++jj) {
+            const int r = 8 * (8 * w + jj) + (lane >> 3);
+            const int c = (lane & 7) ^ ((r >> 1) & 7);
+            const int n = n0 + r < N ? n0 + r : N - 1;
+            wsrc[jj] = static_cast<uint32_t>(n) * K * 2u + c * 16u;
+        }
     } else {
         #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
@@ -387,6 +402,8 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
         uint8_t* xs = lds + slot * kStage;
         if constexpr (j < TM)
             lds_fill16(Xb + static_cast<size_t>(stage_k) * 128 + xsrc[j], xs + 1024 * (w + 4 * j));
+        else if constexpr (F16)
+            lds_fill16(W + static_cast<size_t>(stage_k) * 128 + wsrc[j - TM], xs + kXStage + 1024 * (8 * w + (j - TM)));
         else if constexpr (!Q4)
             lds_fill16(W + static_cast<size_t>(stage_k) * 64 + wsrc[j - TM], xs + kXStage + 1024 * (4 * w + (j - TM)));
         else if constexpr (j - TM < 2)
@@ -402,20 +419,27 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
     // pair S (0, 1) of a stage, MFMA e (0, 1) of the pair: x chunk 4S + 2g + e, W chunk 2S + g
     const uint32_t xrow = lbase + li * 128u, xq = (2u * g) ^ ((li >> 1) & 7u);
     // Q4: bytes 16 S + 8 g .. + 7 of the row: chunk S, its lower or upper half
+    // fp16: as x (the swizzle of rows li and li + 32 is the same)
     const uint32_t wrow = lbase + kXStage + (64u * w + li) * kWRow, wq = Q4 ? (li >> 3) & 1u : g ^ ((li >> 2) & 3u);
     const uint32_t soff = lbase + kScaleAt + (64u * w + li) * 4u;
-    uint32_t xoff[2][2], woff[2];
+    uint32_t xoff[2][2], woff[2], whoff[2][2];
     #pragma unroll
     for (int S = 0; S < 2; ++S) {
         #pragma unroll
-        for (int e = 0; e < 2; ++e) xoff[S][e] = xrow + (((4u * S + e) ^ xq) << 4);
+        for (int e = 0; e < 2; ++e) {
+            xoff[S][e] = xrow + (((4u * S + e) ^ xq) << 4);
+            whoff[S][e] = wrow + (((4u * S + e) ^ xq) << 4);
+        }
         woff[S] = Q4 ? wrow + ((S ^ wq) << 4) + 8u * g : wrow + (((2u * S) ^ wq) << 4);
     }
     // LDS read j (0 .. kReads - 1) of a set: the two W fragments first, then x for the first and
     // the second MFMA of the pair
     auto read_one = [&](Frags<TM>& F, uint32_t slot_bytes, auto Sc, auto jc) {
         constexpr int S = decltype(Sc)::value, j = decltype(jc)::value;
-        if constexpr (j < 2) {
+        if constexpr (F16 && j < kWReads) {
+            const uint32_t a = whoff[S][j % 2] + slot_bytes;
+            MI_LDS_READ16(F.wh[j / 2][j % 2], a, (j / 2) * 32 * kWRow);
+        } else if constexpr (j < 2) {
             const uint32_t a = woff[S] + slot_bytes;
             if constexpr (Q4) {
                 MI_LDS_READ8(F.w4[j], a, j * 32 * kWRow);
@@ -471,7 +495,8 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
     // MFMA n (0 .. kMfmas - 1) of a half stage; consecutive n use different accumulators
     auto mfma_one = [&](const Frags<TM>& F, auto nc) {
         constexpr int n = decltype(nc)::value, c = n / (2 * TM), e = c % 2, u = (n / TM) % 2, t = n % TM;
-        const u32x4 wv = c / 2 ? u32x4{F.wg[u][e][0], F.wg[u][e][1], F.wg[u][e][2], F.wg[u][e][3]}
+        const u32x4 wv = F16 ? F.wh[u][e]
+                       : c / 2 ? u32x4{F.wg[u][e][0], F.wg[u][e][1], F.wg[u][e][2], F.wg[u][e][3]}
                                : u32x4{F.wf[u][e][0], F.wf[u][e][1], F.wf[u][e][2], F.wf[u][e][3]};
         acc[u][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, wv),
                                                           __builtin_bit_cast(half8, F.x[e][t]), acc[u][t], 0, 0, 0);
@@ -487,7 +512,7 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
                           int fill_k, int fill_slot) {
         constexpr bool FILL = decltype(fillc)::value;
         constexpr int nF = FILL ? kLoads : 0;
-        constexpr int A = nF + kReads + 1 + 8;           // fills, reads, wait for W, conversions
+        constexpr int A = nF + kReads + (kConv ? 1 + kConv : 0);   // fills, reads, wait for W, conversions
         static_for<kMfmas>([&](auto nc) {
             constexpr int n = decltype(nc)::value;
             mfma_one(C, nc);
@@ -502,7 +527,9 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
                 } else if constexpr (a == nF + kReads) {
                     // LDS returns in order: the two W reads are back.  The registers are operands
                     // of the wait so that the conversions that read them cannot be moved above it.
-                    if constexpr (Q4)
+                    if constexpr (F16)
+                        ;
+                    else if constexpr (Q4)
                         asm volatile("s_waitcnt lgkmcnt(%4)"
                                      : "+v"(Nx.w4[0]), "+v"(Nx.w4[1]), "+v"(Nx.ws[0]), "+v"(Nx.ws[1])
                                      : "n"(kReads - kWReads) : "memory");
@@ -550,10 +577,12 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
     static_for<kReads>([&](auto jc) { read_one(FA, 0u, std::integral_constant<int, 0>{}, jc); });
     if constexpr (Q4)
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(FA.w4[0]), "+v"(FA.w4[1]), "+v"(FA.ws[0]), "+v"(FA.ws[1]) : : "memory");
+    else if constexpr (F16)
+        MI_WAIT_LGKM(0);
     else
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(FA.w[0]), "+v"(FA.w[1]) : : "memory");
     MI_SCHED_FENCE();
-    static_for<8>([&](auto jc) { convert_one(FA, std::integral_constant<int, 0>{}, jc); });
+    static_for<kConv>([&](auto jc) { convert_one(FA, std::integral_constant<int, 0>{}, jc); });
 
     // Stage i lives in slot i % kStages.  In the middle of stage i every wavefront waits for its
     // own fills of stage i + 1 and meets the others at the barrier; behind it stage i + 1 is
@@ -625,7 +654,7 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
         #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
             float s4[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-            if constexpr (!Q4) {
+            if constexpr (!Q4 && !F16) {
                 s4[0] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].x & 0xFFFFu)));
                 s4[1] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].x >> 16)));
                 s4[2] = __half2float(__ushort_as_half(static_cast<uint16_t>(sc[u][rq].y & 0xFFFFu)));
@@ -710,7 +739,7 @@ bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, co
     if (splits > 1) {
         const long MN = static_cast<long>(M) * N;
         hipLaunchKernelGGL(reduce_partials, dim3(static_cast<unsigned>((MN / 4 + 256) / 256)), dim3(256), 0, s,
-                           partial, splits, KIND == WK_Q4 ? nullptr : static_cast<const uint16_t*>(scale),
+                           partial, splits, KIND == WK_I8 ? static_cast<const uint16_t*>(scale) : nullptr,
                            static_cast<uint16_t*>(out), MN, N);
         if (!MI_HIP_OK(hipGetLastError())) return false;
     }
@@ -727,7 +756,8 @@ bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, co
 inline double estimate_us(int kind, int terms, int tm, int splits, int M, int N, int K, int cus) {
     const long blocks = static_cast<long>((M + 32 * tm - 1) / (32 * tm)) * ((N + kBN - 1) / kBN) * splits;
     const int stages = (K / 64 + splits - 1) / splits;
-    const double stage_us = kind == WK_Q4 ? (terms == 2 ? 0.49 + 0.22 * tm : 0.56 + 0.10 * tm) : 0.27 + 0.10 * tm;
+    const double stage_us = kind == WK_Q4 ? (terms == 2 ? 0.49 + 0.22 * tm : 0.56 + 0.10 * tm)
+                          : kind == WK_F16 ? 0.35 + 0.10 * tm : 0.27 + 0.10 * tm;
     const double block_us = 2.6 + 0.5 * tm + stages * stage_us;
     const long full = blocks / cus, rem = blocks % cus;
     double t = full * 1.56 * block_us + (rem ? (1.0 + 0.56 * rem / cus) * block_us : 0.0);
@@ -823,8 +853,8 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
     // int8: the wide kernel where its estimated time beats that of the 64 x 64 tiles, which are
     // bound either by one tile's serial K loop (about 0.4 us per K-tile, up to 1.3 times that as
     // the chip fills) or by throughput (1.2 to 1.55 ns per tile and K-tile); fitted to measurements
-    const bool wide_fits = kind != WK_F16 && static_cast<double>(M) * K * 2 < 4294967296.0 &&
-                           static_cast<double>(N) * K < 4294967296.0;   // 32-bit byte offsets
+    const bool wide_fits = static_cast<double>(M) * K * 2 < 4294967296.0 &&
+                           static_cast<double>(N) * K * (kind == WK_F16 ? 2 : 1) < 4294967296.0;   // 32-bit byte offsets
     if (kind == WK_Q4) {
         // Q4 weights have the wide kernel only; modes 3 and 11..15 pin it to one slice of K.
         // Mode 4 feeds every weight as the single fp16 number nearest to q * scale (half the
@@ -847,18 +877,21 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
         double wide_us = 0.0;
         int tm = 1, splits = 1;
         // modes 3 and 11..15 pin the plain kernel; slices of K are the library's own choice (mode 0)
-        wide::pick_shape(WK_I8, 1, M, N, K, cus, mode == 0 && workspace ? workspace_bytes : 0, &tm, &splits, &wide_us);
+        wide::pick_shape(kind, 1, M, N, K, cus, mode == 0 && workspace ? workspace_bytes : 0, &tm, &splits, &wide_us);
         const int nk = K / kKT;
         const long t64 = tiles(M, N, 64, 64);
         const double serial = (0.9 + nk * 0.4) * (1.0 + 0.3 * (t64 < 128 ? t64 / 128.0 : 1.0));
         const double bulk = 3.3 + t64 * nk * (nk > 32 ? 0.00155 : 0.0012);
         const double tiled_us = serial > bulk ? serial : bulk;
         if (mode >= 11) tm = mode - 10;
-        if (mode != 0 || wide_us < tiled_us)
+        if (mode != 0 || wide_us < tiled_us) {
+            if (kind == WK_F16)
+                return wide::launch_any<WK_F16, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), splits);
             return wide::launch_any<WK_I8, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), splits);
+        }
     } else if (mode == 3 || mode >= 11) {
-        MI_ERROR_FMT("gemm: mode %d asks for the wide int8 kernel, which does not take kind=%d M=%d N=%d K=%d",
-                     mode, static_cast<int>(kind), M, N, K);
+        MI_ERROR_FMT("gemm: mode %d asks for the wide kernel, whose 32-bit offsets do not reach M=%d N=%d K=%d",
+                     mode, M, N, K);
         return false;
     }
     // 128 x 128 tiles once they fill every CU twice over (two blocks are resident per CU);

@@ -278,6 +278,19 @@ def main():
                     "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                     "frac_hbm": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
             mil.nnopt_unregister_weight(wb)
+        # the same contractions with fp16 weights
+        for (N, K) in ((INTER, H), (H, INTER)):
+            wb = mil.Buffer.from_host(mil.synth_normal_f16(77, 0.02, (N, K)))
+            M = 2048
+            xb = mil.Buffer.from_host(mil.synth_normal_f16(78, 1.0, (M, K)))
+            ob = mil.Buffer(M * N * 2)
+            arr = mil.make_calls([(M, N, K, xb, wb, ob)] * 20)
+            mil.linear_batch(queue, arr)
+            ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 5) / 20
+            flop = 2.0 * M * N * K
+            detail[f"c5_fp16_gemm_M{M}_N{N}_K{K}"] = {
+                "us": round(ms * 1e3, 2), "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 1),
+                "frac_mfma_fp16_peak": round(flop / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)}
         # the same contraction with Q4 weights: exact two-term feed (default) and single rounding (mode 4)
         N, K = INTER, H
         ph, sh = mil.quantize_q4(mil.synth_normal_f16(77, 0.02, (N, K)))

@@ -141,8 +141,8 @@ int   mi_graph_destroy(void* graph);
  * are bit-identical to M = 1 calls (the reference's prefill loop, LF/src/model.cpp:243-250);
  * 2, 3 and 11..15 = as 0 with the kernel choice pinned (tests and tuning: results stay within
  * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel (int8 and fp16
- * weights), 3 = the wide kernel, 10 + t (t = 1..5) = the wide kernel with 32 t rows of x per
- * block; 3 and 10 + t take int8 and Q4 weights and fail for fp16 weights.
+ * weights; fails for Q4), 3 = the wide kernel, 10 + t (t = 1..5) = the wide kernel with 32 t
+ * rows of x per block.
  * Q4 weights: a weight q * scale (4 and 11 significant bits) is not an fp16 number in general.
  * Every mode but 4 feeds it to the matrix cores exactly, as two fp16 terms q * hi + q * lo with
  * scale = hi + lo, and stays within one fp16 step of the batched GEMV.  Mode 4 = as 0, but each

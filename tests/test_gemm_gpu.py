@@ -37,7 +37,7 @@ def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0):
     """tile is the mi_set_gemm_mode value: 0 = the library's own choice, 1 = rows of GEMV,
     2 = the 64 x 64 MFMA kernel, 3 = the wide kernel with its own choice of rows of x per
     block, 4 = Q4 weights rounded to fp16 once, 11..15 = the wide kernel with 32, 64, .. 160 rows
-    of x per block (int8 and Q4)."""
+    of x per block."""
     xb, wb = mil.Buffer.from_host(X), mil.Buffer.from_host(W_host)
     sb = mil.Buffer.from_host(scale_host) if scale_host is not None else None
     if kind == "i8":
@@ -74,9 +74,9 @@ def test_int8_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
     assert np.mean(got == want) > 0.99
 
 
-@pytest.mark.parametrize("tile", [0, 2])
-@pytest.mark.parametrize("M,N,K", [(64, 4864, 896), (256, 896, 4864), (33, 200, 128), (130, 131, 64),
-                                   (2048, 4864, 128)])   # the last one takes the 128 x 128 tiles in mode 0
+@pytest.mark.parametrize("tile", [0, 2, 3, 11, 12, 13, 14, 15])
+@pytest.mark.parametrize("M,N,K", [(64, 4864, 896), (256, 896, 4864), (33, 200, 128), (130, 131, 64), (16, 1536, 576),
+                                   (2048, 4864, 128)])
 def test_fp16_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
     print(f"fp16 gemm M={M} N={N} K={K} tile mode {tile}", flush=True)
     W, X = synth_w(900 + N, N, K), synth_x(901 + M, M, K)
@@ -84,6 +84,20 @@ def test_fp16_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
     want = O.gemm_f16(X, W)
     assert_tolerance(got.view(np.float16), want.view(np.float16))
     assert _ulp_apart(got, want).max() <= 1
+
+
+@pytest.mark.parametrize("tile", [2, 3, 11, 12, 13, 14, 15])
+def test_fp16_gemm_exact_and_repeatable_on_integer_data(queue, tile):
+    """Small integers in both operands: every sum is exact, so the result is that of integer
+    arithmetic whatever the order; and 10 launches of the same call give the same bits."""
+    rng = np.random.default_rng(7)
+    M, N, K = 100, 520, 1024
+    W = rng.integers(-8, 9, (N, K)).astype(np.float16)
+    X = rng.integers(-3, 4, (M, K)).astype(np.float16)
+    want = (X.astype(np.int64) @ W.astype(np.int64).T).astype(np.float16)
+    for _ in range(10):
+        got = _gemm(queue, M, N, K, X, W, None, "f16", tile)
+        assert np.array_equal(got.view(np.float16), want)
 
 
 @pytest.mark.parametrize("tile", [2, 3, 11, 13, 15])
