@@ -33,7 +33,7 @@ const DeviceInfo& device_info();
 // 0 = every GEMV evaluates the reference kernels' sum in their order (bit-exact);
 // 1 = Q4 may use the throughput kernel (same fp32 sum, other order).
 int gemv_mode();
-int gemm_mode();   // 0 auto, 1 batched GEMV, 2 / 3 force the 64 x 64 / 128 x 128 MFMA tile
+int gemm_mode();   // value of mi_set_gemm_mode: 0 auto, 1 rows of GEMV, others pin a GEMM kernel
 
 // M rows of x (stride K) against one W; y rows have stride N.
 struct GemvCall {
@@ -62,8 +62,11 @@ constexpr size_t kArgmaxScratchBytes = 512;
 bool launch_argmax_f16(hipStream_t s, const void* logits, int N, int num_partials, void* token_out, void* scratch);
 
 // gemm.hip: out[M,N] = x[M,K] W^T on MFMA with the dequant fused into the tile load.
-bool gemm_supported(WeightKind kind, int M, int N, int K);
-// workspace: device memory that belongs to stream s (or null): the int8 kernel may cut K into
+// Shapes and pointers the GEMM kernels take (M >= 2, K a multiple of 64, 16-byte aligned x and W).
+bool gemm_supported(WeightKind kind, int M, int N, int K, const void* x, const void* W, const void* scale);
+// Estimated time (us) of the kernel launch_gemm would pick in mode 0.
+double gemm_estimate_us(WeightKind kind, int M, int N, int K, size_t workspace_bytes);
+// workspace: device memory that belongs to stream s (or null): the wide kernel may cut K into
 // slices and park fp32 partial sums there; calls on one stream are ordered, so they can share it.
 bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x,
                  const void* W, const void* scale, void* out, void* workspace, size_t workspace_bytes);

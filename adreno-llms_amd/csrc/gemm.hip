@@ -833,28 +833,55 @@ inline long tiles(int M, int N, int bm, int bn) {
 
 }  // namespace
 
-bool gemm_supported(WeightKind kind, int M, int N, int K) {
-    return (kind == WK_I8 || kind == WK_F16 || kind == WK_Q4) && M >= 16 && N >= 1 && K >= kKT && K % kKT == 0;
+bool gemm_supported(WeightKind kind, int M, int N, int K, const void* x, const void* W, const void* scale) {
+    if (!(kind == WK_I8 || kind == WK_F16 || kind == WK_Q4) || M < 2 || N < 1 || K < kKT || K % kKT != 0) return false;
+    if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(W) % 16) return false;
+    if (kind != WK_F16 && !scale) return false;
+    return kind != WK_Q4 || reinterpret_cast<uintptr_t>(scale) % 4 == 0;
+}
+
+namespace {
+
+bool wide_reaches(WeightKind kind, int M, int N, int K) {     // 32-bit byte offsets
+    return static_cast<double>(M) * K * 2 < 4294967296.0 &&
+           static_cast<double>(N) * K * (kind == WK_F16 ? 2 : 1) < 4294967296.0;
+}
+
+// The 64 x 64 tiles are bound either by one tile's serial K loop (about 0.4 us per K-tile, up to
+// 1.3 times that as the chip fills) or by throughput (1.2 to 1.55 ns per tile and K-tile);
+// fitted to measurements.
+double tiled_estimate_us(int M, int N, int K) {
+    const int nk = K / kKT;
+    const long t64 = tiles(M, N, 64, 64);
+    const double serial = (0.9 + nk * 0.4) * (1.0 + 0.3 * (t64 < 128 ? t64 / 128.0 : 1.0));
+    const double bulk = 3.3 + t64 * nk * (nk > 32 ? 0.00155 : 0.0012);
+    return serial > bulk ? serial : bulk;
+}
+
+}  // namespace
+
+double gemm_estimate_us(WeightKind kind, int M, int N, int K, size_t workspace_bytes) {
+    const int terms = kind == WK_Q4 ? 2 : 1;
+    double wide_us = 1e30;
+    int tm = 1, splits = 1;
+    if (wide_reaches(kind, M, N, K))
+        wide::pick_shape(kind, terms, M, N, K, device_info().cus, workspace_bytes, &tm, &splits, &wide_us);
+    if (kind == WK_Q4) return wide_us;
+    const double tiled_us = tiled_estimate_us(M, N, K);
+    return wide_us < tiled_us ? wide_us : tiled_us;
 }
 
 bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x, const void* W,
                  const void* scale, void* out, void* workspace, size_t workspace_bytes) {
-    if (!gemm_supported(kind, M, N, K)) {
-        MI_ERROR_FMT("gemm: unsupported kind=%d M=%d N=%d K=%d", static_cast<int>(kind), M, N, K);
-        return false;
-    }
-    if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(W) % 16 ||
-        (kind != WK_F16 && !scale) || (kind == WK_Q4 && reinterpret_cast<uintptr_t>(scale) % 4)) {
-        MI_ERROR_FMT("gemm: x and W must be 16-byte aligned; int8 and Q4 need a scale, Q4 a 4-byte aligned one");
+    if (!gemm_supported(kind, M, N, K, x, W, scale)) {
+        MI_ERROR_FMT("gemm: unsupported kind=%d M=%d N=%d K=%d, or x / W not 16-byte aligned, or int8 / Q4 "
+                     "without a (4-byte aligned) scale", static_cast<int>(kind), M, N, K);
         return false;
     }
     const int mode = gemm_mode() == 4 && kind != WK_Q4 ? 0 : gemm_mode();   // mode 4 only concerns Q4 weights
     const int cus = device_info().cus;
-    // int8: the wide kernel where its estimated time beats that of the 64 x 64 tiles, which are
-    // bound either by one tile's serial K loop (about 0.4 us per K-tile, up to 1.3 times that as
-    // the chip fills) or by throughput (1.2 to 1.55 ns per tile and K-tile); fitted to measurements
-    const bool wide_fits = static_cast<double>(M) * K * 2 < 4294967296.0 &&
-                           static_cast<double>(N) * K * (kind == WK_F16 ? 2 : 1) < 4294967296.0;   // 32-bit byte offsets
+    // int8 and fp16: the wide kernel where its estimated time beats that of the 64 x 64 tiles
+    const bool wide_fits = wide_reaches(kind, M, N, K);
     if (kind == WK_Q4) {
         // Q4 weights have the wide kernel only; modes 3 and 11..15 pin it to one slice of K.
         // Mode 4 feeds every weight as the single fp16 number nearest to q * scale (half the
@@ -878,11 +905,7 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
         int tm = 1, splits = 1;
         // modes 3 and 11..15 pin the plain kernel; slices of K are the library's own choice (mode 0)
         wide::pick_shape(kind, 1, M, N, K, cus, mode == 0 && workspace ? workspace_bytes : 0, &tm, &splits, &wide_us);
-        const int nk = K / kKT;
-        const long t64 = tiles(M, N, 64, 64);
-        const double serial = (0.9 + nk * 0.4) * (1.0 + 0.3 * (t64 < 128 ? t64 / 128.0 : 1.0));
-        const double bulk = 3.3 + t64 * nk * (nk > 32 ? 0.00155 : 0.0012);
-        const double tiled_us = serial > bulk ? serial : bulk;
+        const double tiled_us = tiled_estimate_us(M, N, K);
         if (mode >= 11) tm = mode - 10;
         if (mode != 0 || wide_us < tiled_us) {
             if (kind == WK_F16)

@@ -225,6 +225,18 @@ void mi_set_gemv_mode(int mode) { g_gemv_mode = mode; }
 
 // ---- hot path --------------------------------------------------------------------
 
+// M > 1: a real contraction goes to the MFMA GEMM.  Every batch in mode 1, and shapes the GEMM
+// does not take, run the GEMV once per row of x, as the reference's quantised prefill does; so
+// do batches below 16 rows while that is estimated to be faster (each GEMV row streams W again:
+// about bytes / 6.6 TB/s, or 1 us when W stays in the caches).
+static bool takes_gemm(hipStream_t s, const Entry& e, int M, int N, int K, const void* x, const void* W) {
+    if (M < 2 || g_gemm_mode == 1 || !gemm_supported(e.kind, M, N, K, x, W, e.scale)) return false;
+    if (M >= 16 || g_gemm_mode != 0) return true;
+    const double w_bytes = static_cast<double>(N) * K * (e.kind == WK_F16 ? 2.0 : e.kind == WK_I8 ? 1.0 : 0.5625);
+    const double row_us = w_bytes / 6.6e6 > 1.0 ? w_bytes / 6.6e6 : 1.0;
+    return gemm_estimate_us(e.kind, M, N, K, workspace_of(s) ? kWorkspaceBytes : 0) < 2.5 + M * row_us;
+}
+
 int mi_linear(void* stream, int M, int N, int K, const void* x, const void* W, void* out) {
     if (!ensure_init()) return 0;
     if (M <= 0 || N <= 0 || K <= 0 || !x || !W || !out) {
@@ -233,9 +245,7 @@ int mi_linear(void* stream, int M, int N, int K, const void* x, const void* W, v
     }
     Entry e;
     if (!resolve("mi_linear", W, N, K, &e)) return 0;
-    // M > 1: a real contraction goes to the MFMA GEMM; small batches, and every batch in
-    // mode 1, run the GEMV once per row of x, as the reference's quantised prefill does.
-    if (M >= 16 && g_gemm_mode != 1 && gemm_supported(e.kind, M, N, K))
+    if (takes_gemm(as_stream(stream), e, M, N, K, x, W))
         return launch_gemm(as_stream(stream), e.kind, M, N, K, x, W, e.scale, out, workspace_of(as_stream(stream)),
                            kWorkspaceBytes) ? 1 : 0;
     GemvCall c;
@@ -281,7 +291,8 @@ int mi_linear_batch(void* stream, const mi_linear_call* calls, int n) {
         const mi_linear_call& c0 = calls[i];
         Entry e0;
         const bool groupable = c0.M >= 1 && c0.M < 16 && c0.N > 0 && c0.K > 0 && c0.x && c0.W && c0.out &&
-                               resolve("mi_linear_batch", c0.W, c0.N, c0.K, &e0);
+                               resolve("mi_linear_batch", c0.W, c0.N, c0.K, &e0) &&
+                               !takes_gemm(as_stream(stream), e0, c0.M, c0.N, c0.K, c0.x, c0.W);
         if (!groupable) {
             if (!mi_linear(stream, c0.M, c0.N, c0.K, c0.x, c0.W, c0.out)) return i;
             ++i;

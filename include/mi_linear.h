@@ -136,8 +136,10 @@ void* mi_graph_end(void* stream);              /* returns an executable graph or
 int   mi_graph_launch(void* graph, void* stream);
 int   mi_graph_destroy(void* graph);
 
-/* Selects how M > 1 is computed for a quantised W: 0 (default) = MFMA GEMM with fused
- * dequant for M >= 16 and batched GEMV below; 1 = always the batched GEMV, whose rows
+/* Selects how M > 1 is computed: 0 (default) = MFMA GEMM with fused dequant for M >= 16, and
+ * for 2 <= M < 16 where it is estimated to beat M rows of GEMV (each row streams W again; e.g. an
+ * lm_head from M = 2, an MLP projection from M = 4 to 10); K not a multiple of 64 or operands
+ * not 16-byte aligned always take the batched GEMV; 1 = always the batched GEMV, whose rows
  * are bit-identical to M = 1 calls (the reference's prefill loop, LF/src/model.cpp:243-250);
  * 2, 3 and 11..15 = as 0 with the kernel choice pinned (tests and tuning: results stay within
  * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel (int8 and fp16

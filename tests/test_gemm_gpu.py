@@ -220,6 +220,31 @@ def test_q4_gemm_tiny_scales_keep_fp16_subnormals(queue):
     assert _ulp_apart(got, want).max() <= 1
 
 
+@pytest.mark.parametrize("kind", ["i8", "q4", "f16"])
+@pytest.mark.parametrize("tile", [0, 2, 3])
+@pytest.mark.parametrize("M", [2, 5, 15])
+@pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (130, 576)])
+def test_batches_below_16_rows(queue, kind, tile, M, N, K):
+    """2 <= M < 16: mode 0 picks the GEMM or M rows of GEMV by estimated time; either way, and
+    with the GEMM kernels forced, the result is within one fp16 step of the rows of GEMV."""
+    if kind == "q4" and tile == 2:
+        pytest.skip("the 64 x 64 tiles do not take Q4 weights")
+    W, X = synth_w(2700 + N, N, K), synth_x(2800 + M, M, K)
+    if kind == "i8":
+        q, s = mil.quantize_int8(W)
+        got, want = _gemm(queue, M, N, K, X, q, s, "i8", tile), O.gemm_i8(X, q, s.view(np.uint16))
+    elif kind == "q4":
+        p, s = mil.quantize_q4(W)
+        got, want = _gemm(queue, M, N, K, X, p, s, "q4", tile), O.gemm_q4(X, p, s.view(np.uint16))
+    else:
+        got, want = _gemm(queue, M, N, K, X, W, None, "f16", tile), O.gemm_f16(X, W)
+    assert_tolerance(got.view(np.float16), want.view(np.float16))
+    # (rows of GEMV with Q4 weights may come from the throughput kernel of the default GEMV mode,
+    # whose bar is the stated tolerance)
+    if not (kind == "q4" and tile == 0):
+        assert _ulp_apart(got, want).max() <= 1
+
+
 @pytest.mark.parametrize("tile", [3, 4, 11, 13, 15])
 def test_q4_gemm_exact_on_integer_data(queue, tile):
     # power-of-two scales and small integer x: every product and partial sum is exact
