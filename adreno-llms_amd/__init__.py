@@ -61,6 +61,7 @@ _SIGNATURES = {
     "mi_decoder_step": (_i, [_vp, _vp]),
     "mi_decoder_read": (_i, [_vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
     "mi_decoder_logits": (_vp, [_vp]),
+    "mi_decoder_buffer": (_vp, [_vp, _i]),
     "mi_argmax_f16": (_i, [_vp, _vp, _i, _i, _vp]),
     "mi_linear_argmax": (_i, [_vp, _i, _i, _vp, _vp, _vp, _i, _vp]),
     "mi_set_gemm_mode": (None, [_i]),

@@ -15,7 +15,10 @@ SOURCES = ["runtime.hip", "gemv.hip", "gemm.hip", "argmax.hip", "decode.hip", "q
 # may be fused, or results stop being bit-identical to the reference evaluation order.
 # The packed-fp32 feature is switched off for device code on purpose.
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-Wall", "-Wno-unused-result"]
-DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# (fp32 divide and square root correctly rounded: hipcc's default, spelled out because the
+#  decode-step kernels rely on it for bit-identical results)
+DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          "-fhip-fp32-correctly-rounded-divide-sqrt"]
 
 
 def build(verbose=True, extra=()):

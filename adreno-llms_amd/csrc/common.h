@@ -22,7 +22,9 @@
 namespace mi {
 
 enum WeightKind : int { WK_F16 = 0, WK_Q4 = 4, WK_I8 = 8 };
-enum Epilogue : int { EPI_STORE = 0, EPI_ADD = 1 };
+// EPI_SWIGLU: two segments, gate and up, of equal N: y_gate[n] = swiglu(fp16(gate row n), fp16(up row n)),
+// the unfused sequence of two GEMVs and the element-wise kernel; y_up is not written.
+enum Epilogue : int { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2 };
 
 struct DeviceInfo {
     int  device = -1;
@@ -44,6 +46,10 @@ struct GemvCall {
     int M = 1, N = 0, K = 0;
     WeightKind kind = WK_F16;
     Epilogue   epi = EPI_STORE;
+    // Decode-step fusions (no counterpart at the C boundary):
+    const void* norm_w = nullptr; // fp16 [K]: x is RMS-normalised with these weights first (M = 1, see gemv_takes_norm)
+    float       norm_eps = 0.0f;
+    bool        add_rounded = false;  // EPI_ADD: y = fp16(fp16(product) + y), the unfused GEMV-then-add sequence
 };
 
 // gemv.hip
@@ -51,10 +57,20 @@ constexpr int kMaxSegments = 4;
 bool launch_gemv(hipStream_t s, const GemvCall& c);
 // n <= kMaxSegments calls that share x, K, M, weight kind and epilogue, as one launch.
 bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n);
+bool gemv_takes_norm(WeightKind kind, int K);    // GemvCall::norm_w is supported for this kind and K
+bool gemv_takes_swiglu(WeightKind kind, int K);  // EPI_SWIGLU is supported for this kind and K
 bool launch_gate_up_silu(hipStream_t s, WeightKind kind, int N, int K, const void* x,
                          const void* Wg, const void* sg, const void* Wu, const void* su, void* out);
 bool launch_dequant_int8(hipStream_t s, const void* q, const void* scale, int N, int K, void* w16);
 bool launch_unpack_q4(hipStream_t s, const void* p, int N, int K, void* w8);
+
+// runtime.hip: n <= kMaxSegments projections of one x (M = 1) as one GEMV launch, weight kinds and
+// scales from the registry, with the decode-step fusions of GemvCall: the RMSNorm of x ahead
+// (norm_w != null; all W of a kind and K that gemv_takes_norm accepts), the unfused residual
+// add behind (EPI_ADD: y[i] = fp16(fp16(W[i] x) + y[i])) or the SwiGLU of a gate / up pair (EPI_SWIGLU).
+bool fused_gemv(hipStream_t s, int n, const int* N, int K, const void* x, const void* const* W, void* const* y,
+                const void* norm_w, float norm_eps, Epilogue epi);
+bool fused_gemv_kind(const void* W, int N, int K, WeightKind* kind);   // kind W is registered as (fp16 if not)
 
 // argmax.hip: index of the greatest of N fp16 values, ties as the reference's two argmax kernels break them.
 // scratch: kArgmaxScratchBytes of device memory that belongs to stream s, or null (then one block does all the work).

@@ -1,6 +1,7 @@
 // A Qwen2-shaped greedy decode step that stays on the device: the small kernels that sit between
 // the projections (QW/kernels/{embedding,rmsnorm,bias_add,rope,attention,mlp,utils}.cl), the
-// projections themselves through mi_linear / mi_linear_batch, and the argmax.  Graph of a step:
+// projections themselves as GEMV launches that also carry the RMSNorm ahead of them or the
+// residual add behind them, and the argmax.  Graph of a step:
 // QW/src/model.cpp:243-376, QW/src/layers/attention.cpp:336-674, QW/src/layers/mlp.cpp:97-237.
 //
 // Position and token live in device memory (the reference's counter buffer, QW/src/model.cpp:
@@ -40,14 +41,11 @@ __global__ void embed_kernel(const uint16_t* __restrict__ embed, const State* __
 
 // out[c] = fp16((x[c] * inv) * w[c]), inv = 1 / sqrt(mean(x^2) + eps); the sum of squares runs
 // over 64 work-items in float4 strides and a 32..1 tree (QW/kernels/rmsnorm.cl).  One wavefront.
-// With add != null the residual add that precedes the norm in the step runs first, in the same
-// launch: x[c] = fp16(x[c] + add[c]) (QW/kernels/utils.cl element_add), then the norm of the
-// rounded x, exactly as two launches would compute it.
-__global__ __launch_bounds__(64) void rmsnorm_kernel(uint16_t* __restrict__ x, const uint16_t* __restrict__ add,
-                                                     const uint16_t* __restrict__ w, uint16_t* __restrict__ out,
-                                                     int cols, float eps) {
-    // Work-item lid owns the float4 groups lid, lid + 64, ...: it adds, squares and normalises the
-    // same elements, so x, add and w are read once, all loads are in flight together, and the
+// Used where the norm cannot ride in the projection's own launch (see mi_decoder_step).
+__global__ __launch_bounds__(64) void rmsnorm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                     uint16_t* __restrict__ out, int cols, float eps) {
+    // Work-item lid owns the float4 groups lid, lid + 64, ...: it squares and normalises the
+    // same elements, so x and w are read once, all loads are in flight together, and the
     // kernel costs one memory round trip.  Up to kGroups groups per work-item live in registers
     // (cols <= 256 kGroups); the tail that is not a whole group, and longer rows, go through memory.
     constexpr int kGroups = 8;
@@ -61,12 +59,6 @@ __global__ __launch_bounds__(64) void rmsnorm_kernel(uint16_t* __restrict__ x, c
         if (c4 < c4n) {
             xv[g] = *reinterpret_cast<const u16x4*>(x + 4 * c4);
             wv[g] = *reinterpret_cast<const u16x4*>(w + 4 * c4);
-            if (add) {
-                const u16x4 av = *reinterpret_cast<const u16x4*>(add + 4 * c4);
-                #pragma unroll
-                for (int e = 0; e < 4; ++e) xv[g][e] = f_h(h_f(xv[g][e]) + h_f(av[e]));
-                *reinterpret_cast<u16x4*>(x + 4 * c4) = xv[g];
-            }
         }
     }
     #pragma unroll
@@ -83,14 +75,7 @@ __global__ __launch_bounds__(64) void rmsnorm_kernel(uint16_t* __restrict__ x, c
     for (int c4 = lid + 64 * kGroups; c4 < c4n; c4 += 64) {           // rows longer than the registers hold
         float v[4];
         #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            v[e] = h_f(x[4 * c4 + e]);
-            if (add) {
-                const uint16_t r = f_h(v[e] + h_f(add[4 * c4 + e]));
-                x[4 * c4 + e] = r;
-                v[e] = h_f(r);
-            }
-        }
+        for (int e = 0; e < 4; ++e) v[e] = h_f(x[4 * c4 + e]);
         float d = v[0] * v[0];
         d = fmaf(v[1], v[1], d);
         d = fmaf(v[2], v[2], d);
@@ -98,12 +83,7 @@ __global__ __launch_bounds__(64) void rmsnorm_kernel(uint16_t* __restrict__ x, c
         acc = acc + d;
     }
     for (int c = c4n * 4 + lid; c < cols; c += 64) {                    // cols not a multiple of 4
-        float v = h_f(x[c]);
-        if (add) {
-            const uint16_t r = f_h(v + h_f(add[c]));
-            x[c] = r;
-            v = h_f(r);
-        }
+        const float v = h_f(x[c]);
         acc = fmaf(v, v, acc);
     }
     #pragma unroll
@@ -112,7 +92,9 @@ __global__ __launch_bounds__(64) void rmsnorm_kernel(uint16_t* __restrict__ x, c
         acc = acc + o;
     }
     const float total = __shfl(acc, 0, 64);
-    const float inv = rcp_rn(__fsqrt_rn(__fdiv_rn(total, static_cast<float>(cols)) + eps));
+    // sqrtf is the correctly rounded one (-fhip-fp32-correctly-rounded-divide-sqrt); the
+    // __fsqrt_rn intrinsic is not, despite its name: it is off by an ulp for one input in six
+    const float inv = rcp_rn(sqrtf(__fdiv_rn(total, static_cast<float>(cols)) + eps));
     #pragma unroll
     for (int g = 0; g < kGroups; ++g) {
         const int c4 = lid + 64 * g;
@@ -254,7 +236,7 @@ struct Decoder {
     const void* lm_head = nullptr;
     // device memory owned by the decoder
     uint16_t *kc = nullptr, *vc = nullptr, *cosT = nullptr, *sinT = nullptr;
-    uint16_t *h = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *proj = nullptr;
+    uint16_t *h = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr;
     uint16_t *gate = nullptr, *up = nullptr, *logits = nullptr;
     State* st = nullptr;
     std::vector<void*> owned;
@@ -314,7 +296,7 @@ void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* 
               dev_alloc(d, &d->sinT, static_cast<size_t>(c.max_pos) * D * 2) &&
               dev_alloc(d, &d->h, c.hidden * 2) && dev_alloc(d, &d->xn, c.hidden * 2) && dev_alloc(d, &d->q, qd * 2) &&
               dev_alloc(d, &d->k, kvd * 2) && dev_alloc(d, &d->v, kvd * 2) && dev_alloc(d, &d->attn, qd * 2) &&
-              dev_alloc(d, &d->proj, c.hidden * 2) && dev_alloc(d, &d->gate, c.inter * 2) &&
+              dev_alloc(d, &d->gate, c.inter * 2) &&
               dev_alloc(d, &d->up, c.inter * 2) && dev_alloc(d, &d->logits, static_cast<size_t>(c.vocab) * 2) &&
               dev_alloc(d, &d->st, sizeof(State));
     if (ok) {
@@ -386,6 +368,22 @@ int mi_decoder_read(void* dec, void* stream, int* pos, int* token) {
 
 const void* mi_decoder_logits(void* dec) { return dec ? static_cast<Decoder*>(dec)->logits : nullptr; }
 
+const void* mi_decoder_buffer(void* dec, int which) {
+    auto* d = static_cast<Decoder*>(dec);
+    if (!d) return nullptr;
+    switch (which) {
+        case 0: return d->h;
+        case 1: return d->q;
+        case 2: return d->k;
+        case 3: return d->v;
+        case 4: return d->attn;
+        case 5: return d->gate;
+        case 6: return d->cosT;
+        case 7: return d->sinT;
+        default: return nullptr;
+    }
+}
+
 int mi_decoder_step(void* dec, void* stream) {
     auto* d = static_cast<Decoder*>(dec);
     if (!d) return 0;
@@ -394,21 +392,54 @@ int mi_decoder_step(void* dec, void* stream) {
     const int Hd = c.hidden, D = c.head_dim, qd = c.n_heads * D, kvd = c.n_kv_heads * D;
     const float scale = 1.0f / sqrtf(static_cast<float>(D));
     auto launched = [] { return MI_HIP_OK(hipGetLastError()); };
-    // x (+= residual, if given), then out = rmsnorm(x) * w
-    auto rmsnorm = [&](uint16_t* x, const uint16_t* residual, const void* w, uint16_t* out) {
-        hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(64), 0, s, x, residual, static_cast<const uint16_t*>(w), out, Hd,
-                           c.rms_eps);
-        return launched();
+    // Projections of rmsnorm(h) * w.  The norm rides in the GEMV launch where the weights allow it
+    // (every wavefront repeats it while its first weights are in flight); otherwise it is a
+    // launch of its own into xn.
+    // With swiglu set (gate and up projection), y[0] receives swiglu(gate, up) and the SwiGLU
+    // rides in the same launch too where it can.
+    auto norm_linear = [&](const void* w, int n, const int* N, const void* const* W, void* const* y, bool swiglu) {
+        WeightKind kind = WK_F16, k0 = WK_F16;
+        bool fuse = true;
+        for (int i = 0; i < n; ++i) {
+            if (!fused_gemv_kind(W[i], N[i], Hd, &kind)) return false;
+            if (i == 0) k0 = kind;
+            fuse = fuse && kind == k0 && gemv_takes_norm(kind, Hd);
+        }
+        if (fuse && swiglu && gemv_takes_swiglu(k0, Hd)) return fused_gemv(s, n, N, Hd, d->h, W, y, w, c.rms_eps, EPI_SWIGLU);
+        if (fuse) {
+            if (!fused_gemv(s, n, N, Hd, d->h, W, y, w, c.rms_eps, EPI_STORE)) return false;
+        } else {
+            hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(64), 0, s, d->h, static_cast<const uint16_t*>(w), d->xn, Hd,
+                               c.rms_eps);
+            if (!launched()) return false;
+            mi_linear_call calls[kMaxSegments];
+            for (int i = 0; i < n; ++i) calls[i] = mi_linear_call{1, N[i], Hd, d->xn, W[i], y[i]};
+            if (mi_linear_batch(stream, calls, n) != n) return false;
+        }
+        if (swiglu) {
+            hipLaunchKernelGGL(swiglu_kernel, dim3((N[0] + 255) / 256), dim3(256), 0, s, static_cast<uint16_t*>(y[0]),
+                               static_cast<const uint16_t*>(y[1]), N[0]);
+            return launched();
+        }
+        return true;
+    };
+    // h = fp16(h + fp16(W x)): the projection and the element-wise add that follows it
+    // (QW/kernels/utils.cl element_add), one launch
+    auto linear_into_h = [&](int K, const void* x, const void* W) {
+        const int N1[1] = {Hd};
+        const void* const W1[1] = {W};
+        void* const y1[1] = {d->h};
+        return fused_gemv(s, 1, N1, K, x, W1, y1, nullptr, 0.0f, EPI_ADD);
     };
     hipLaunchKernelGGL(embed_kernel, dim3(1), dim3(256), 0, s, static_cast<const uint16_t*>(d->embed), d->st, d->h, Hd, c.vocab);
     if (!launched()) return 0;
     for (int l = 0; l < c.n_layers; ++l) {
-        // the previous layer's down-projection residual is added here, ahead of this layer's first norm
-        if (!rmsnorm(d->h, l ? d->proj : nullptr, d->in_norm[l], d->xn)) return 0;
-        const mi_linear_call qkv[3] = {{1, qd, Hd, d->xn, d->wq[l], d->q},
-                                       {1, kvd, Hd, d->xn, d->wk[l], d->k},
-                                       {1, kvd, Hd, d->xn, d->wv[l], d->v}};
-        if (mi_linear_batch(stream, qkv, 3) != 3) return 0;
+        {
+            const int N3[3] = {qd, kvd, kvd};
+            const void* const W3[3] = {d->wq[l], d->wk[l], d->wv[l]};
+            void* const y3[3] = {d->q, d->k, d->v};
+            if (!norm_linear(d->in_norm[l], 3, N3, W3, y3, false)) return 0;
+        }
         uint16_t* kc = d->kc + static_cast<size_t>(l) * c.max_pos * kvd;
         uint16_t* vc = d->vc + static_cast<size_t>(l) * c.max_pos * kvd;
         const int pairs = (c.n_heads + c.n_kv_heads) * D / 2;
@@ -421,18 +452,22 @@ int mi_decoder_step(void* dec, void* stream) {
         hipLaunchKernelGGL(attention_kernel, dim3(c.n_heads), dim3(at), static_cast<size_t>(c.max_pos) * 6, s, d->q, kc, vc,
                            d->attn, d->st, c.n_heads, c.n_kv_heads, D, c.max_pos, scale);
         if (!launched()) return 0;
-        if (!mi_linear(stream, 1, Hd, qd, d->attn, d->wo[l], d->proj)) return 0;
-        if (!rmsnorm(d->h, d->proj, d->post_norm[l], d->xn)) return 0;          // h += o-projection, then the norm
-        const mi_linear_call gu[2] = {{1, c.inter, Hd, d->xn, d->wgate[l], d->gate}, {1, c.inter, Hd, d->xn, d->wup[l], d->up}};
-        if (mi_linear_batch(stream, gu, 2) != 2) return 0;
-        hipLaunchKernelGGL(swiglu_kernel, dim3((c.inter + 255) / 256), dim3(256), 0, s, d->gate, d->up, c.inter);
-        if (!launched()) return 0;
-        if (!mi_linear(stream, 1, Hd, c.inter, d->gate, d->wdown[l], d->proj)) return 0;
+        if (!linear_into_h(qd, d->attn, d->wo[l])) return 0;
+        {
+            const int N2[2] = {c.inter, c.inter};
+            const void* const W2[2] = {d->wgate[l], d->wup[l]};
+            void* const y2[2] = {d->gate, d->up};
+            if (!norm_linear(d->post_norm[l], 2, N2, W2, y2, true)) return 0;
+        }
+        if (!linear_into_h(c.inter, d->gate, d->wdown[l])) return 0;
     }
-    if (!rmsnorm(d->h, d->proj, d->final_norm, d->xn)) return 0;                // the last residual add, then the final norm
-    if (!mi_linear_argmax(stream, c.vocab, Hd, d->xn, d->lm_head, d->logits, 32,
-                          reinterpret_cast<char*>(d->st) + offsetof(State, next)))
-        return 0;
+    {
+        const int N1[1] = {c.vocab};
+        const void* const W1[1] = {d->lm_head};
+        void* const y1[1] = {d->logits};
+        if (!norm_linear(d->final_norm, 1, N1, W1, y1, false)) return 0;
+    }
+    if (!mi_argmax_f16(stream, d->logits, c.vocab, 32, reinterpret_cast<char*>(d->st) + offsetof(State, next))) return 0;
     hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->st);
     return launched() ? 1 : 0;
 }

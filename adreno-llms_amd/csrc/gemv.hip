@@ -56,7 +56,17 @@ struct SegList {
     Seg s[kMaxSegments];
     int nseg;
     int nbatch;      // row batches of all segments
+    const uint16_t* norm_w;   // not null: x is RMS-normalised with these weights before use
+    float norm_eps;
+    int add_rounded;          // EPI_ADD: the product is rounded to fp16 before the residual is added
 };
+
+// EPI_ADD, the two forms: the fused one of the reference's residual kernels (one rounding), and
+// the unfused sequence GEMV, then element-wise add of two fp16 vectors (two roundings).
+__device__ __forceinline__ float add_residual(float sum, float s, float res, bool scaled, int rounded) {
+    if (rounded) return h_f(f_h(scaled ? sum * s : sum)) + res;
+    return scaled ? fmaf(sum, s, res) : sum + res;
+}
 
 __device__ __forceinline__ float lo_f(uint32_t p) {
     return __half2float(__ushort_as_half(static_cast<unsigned short>(p & 0xffffu)));
@@ -273,6 +283,7 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     const int step = nw * GB;
     Group g0, g1;
     fetch_group(g0, rb);
+    if constexpr (EPI == EPI_SWIGLU) fetch(g1.b[0], rb + L.s[1].first);
 
     uint32_t xr[NIT][XD];
     #pragma unroll
@@ -284,7 +295,50 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
         }
     }
 
-    auto consume = [&](const Batch& b) {
+    // RMSNorm of x in place of a kernel of its own (QW/kernels/rmsnorm.cl: 64 lanes, each summing
+    // the squares of elements 4 lane + 256 j, the same tree as the GEMV's, then
+    // fp16((x * inv) * w)): the virtual lanes of this kernel own exactly those elements, so every
+    // wavefront repeats the sum in the reference's order while its first weights are in flight.
+    if constexpr (T::EPV == 4) {
+        if (L.norm_w) {
+            uint32_t nw[NIT][XD];
+            #pragma unroll
+            for (int j = 0; j < NIT; ++j)
+                load_dwords<XD, false>(nw[j], L.norm_w + (j * EIT + koff < KT ? j * EIT + koff : koff));
+            float part[VL];
+            #pragma unroll
+            for (int v = 0; v < VL; ++v) part[v] = 0.0f;
+            #pragma unroll
+            for (int j = 0; j < NIT; ++j) {
+                if (j * EIT + koff < KT) {
+                    #pragma unroll
+                    for (int v = 0; v < VL; ++v) {
+                        const float v0 = lo_f(xr[j][2 * v]), v1 = hi_f(xr[j][2 * v]);
+                        const float v2 = lo_f(xr[j][2 * v + 1]), v3 = hi_f(xr[j][2 * v + 1]);
+                        float d = v0 * v0;
+                        d = fmaf(v1, v1, d);
+                        d = fmaf(v2, v2, d);
+                        d = fmaf(v3, v3, d);
+                        part[v] = part[v] + d;
+                    }
+                }
+            }
+            const float total = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(reduce_row<VL>(part))));
+            // (sqrtf: correctly rounded under -fhip-fp32-correctly-rounded-divide-sqrt, which __fsqrt_rn is not)
+            const float inv = __fdiv_rn(1.0f, sqrtf(__fdiv_rn(total, static_cast<float>(KT)) + L.norm_eps));
+            #pragma unroll
+            for (int j = 0; j < NIT; ++j) {
+                #pragma unroll
+                for (int i = 0; i < XD; ++i) {
+                    const uint32_t lo = f_h((lo_f(xr[j][i]) * inv) * lo_f(nw[j][i]));
+                    const uint32_t hi = f_h((hi_f(xr[j][i]) * inv) * hi_f(nw[j][i]));
+                    xr[j][i] = lo | (hi << 16);
+                }
+            }
+        }
+    }
+
+    auto row_sum = [&](const Batch& b) {
         float acc[VL];
         #pragma unroll
         for (int v = 0; v < VL; ++v) acc[v] = 0.0f;
@@ -297,14 +351,40 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
                     acc[v] = vlane_step<KIND>(acc[v], &b.w[j][v * T::BPV / 4], &xr[j][v * T::EPV / 2], sf, cst);
             }
         }
-        const float sum = reduce_row<VL>(acc);
+        return reduce_row<VL>(acc);
+    };
+
+    if constexpr (EPI == EPI_SWIGLU) {
+        // g0 holds row batch rb of the gate matrix (segment 0), g1 the same rows of the up
+        // matrix (segment 1); the gate and up values are rounded to fp16 as two GEMVs would
+        // store them, then gate[n] = fp16((g * sigmoid(g)) * u)  (QW/kernels/mlp.cl swiglu_inplace)
+        static_assert(!PIPE && KIND != WK_Q4, "one batch pair at a time");
+        while (true) {
+            const float sg_ = row_sum(g0.b[0]), su_ = row_sum(g1.b[0]);
+            if (g == 0 && g0.b[0].yoff >= 0) {
+                const float sgs = KIND == WK_I8 ? sg_ * h_f(g0.b[0].s[0]) : sg_;
+                const float sus = KIND == WK_I8 ? su_ * h_f(g1.b[0].s[0]) : su_;
+                const float gv = h_f(f_h(sgs)), uv = h_f(f_h(sus));
+                const float sig = __fdiv_rn(1.0f, 1.0f + exp_poly(-gv));
+                g0.b[0].ybase[g0.b[0].yoff] = f_h((gv * sig) * uv);
+            }
+            rb += nw;
+            if (rb >= L.nbatch) break;
+            fetch(g0.b[0], rb);
+            fetch(g1.b[0], rb + L.s[1].first);
+        }
+        return;
+    }
+
+    auto consume = [&](const Batch& b) {
+        const float sum = row_sum(b);
         if (g == 0 && b.yoff >= 0) {
             float out;
             if constexpr (KIND == WK_I8) {
                 const float s = h_f(b.s[0]);
-                out = EPI == EPI_ADD ? fmaf(sum, s, h_f(b.res)) : sum * s;
+                out = EPI == EPI_ADD ? add_residual(sum, s, h_f(b.res), true, L.add_rounded) : sum * s;
             } else {
-                out = EPI == EPI_ADD ? sum + h_f(b.res) : sum;
+                out = EPI == EPI_ADD ? add_residual(sum, 1.0f, h_f(b.res), false, L.add_rounded) : sum;
             }
             b.ybase[b.yoff] = f_h(out);
         }
@@ -461,7 +541,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
         acc = add_from_above<2>(acc);
         acc = add_from_above<1>(acc);
         if (g == 0 && b.yoff >= 0) {
-            const float out = EPI == EPI_ADD ? acc + h_f(b.res) : acc;
+            const float out = EPI == EPI_ADD ? add_residual(acc, 1.0f, h_f(b.res), false, L.add_rounded) : acc;
             b.ybase[b.yoff] = f_h(out);
         }
     };
@@ -548,9 +628,9 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict_
             float out;
             if constexpr (KIND == WK_I8) {
                 const float s = h_f(sg.sc[row]);
-                out = EPI == EPI_ADD ? fmaf(sum, s, h_f(*yp)) : sum * s;
+                out = EPI == EPI_ADD ? add_residual(sum, s, h_f(*yp), true, L.add_rounded) : sum * s;
             } else {
-                out = EPI == EPI_ADD ? sum + h_f(*yp) : sum;
+                out = EPI == EPI_ADD ? add_residual(sum, 1.0f, h_f(*yp), false, L.add_rounded) : sum;
             }
             *yp = f_h(out);
         }
@@ -682,6 +762,9 @@ Plan make_plan(const GemvCall* calls, int n, int vl) {
     }
     p.L.nseg = n;
     p.L.nbatch = first;
+    p.L.norm_w = static_cast<const uint16_t*>(calls[0].norm_w);
+    p.L.norm_eps = calls[0].norm_eps;
+    p.L.add_rounded = calls[0].add_rounded ? 1 : 0;
     const int cap = resident_waves();
     int waves = first;
     p.pipe = false;
@@ -727,6 +810,30 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
         }
     }
 #undef MI_FIXED
+    return MI_HIP_OK(hipGetLastError());
+}
+
+// Gate and up projection with the SwiGLU behind them: calls[0] = gate, calls[1] = up.  A
+// wavefront takes the same row batch of both matrices, so the launch has as many batches as one
+// matrix; the kernels that keep x in registers only, without the pipelined variant.
+template <int KIND, int VL>
+bool launch_swiglu_vl(hipStream_t s, const GemvCall* calls) {
+    Plan p = make_plan(calls, 2, VL);
+    p.L.nbatch = p.L.s[1].first;
+    const int cap = resident_waves();
+    const int waves = p.L.nbatch < cap ? p.L.nbatch : cap;
+    p.grid = dim3((waves + kWavesPerBlock - 1) / kWavesPerBlock, 1, 1);
+    const auto* x = static_cast<const uint16_t*>(calls[0].x);
+#define MI_SWIGLU(KT) \
+    case KT: hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI_SWIGLU, false, 1>), p.grid, dim3(kBlock), 0, s, x, p.L); break;
+    switch (calls[0].K) {
+        MI_SWIGLU(576)
+        MI_SWIGLU(896)
+        MI_SWIGLU(1024)
+        MI_SWIGLU(1536)
+        default: MI_ERROR_FMT("gemv: no SwiGLU epilogue for K=%d", calls[0].K); return false;
+    }
+#undef MI_SWIGLU
     return MI_HIP_OK(hipGetLastError());
 }
 
@@ -789,6 +896,15 @@ bool check_call(const GemvCall& c) {
 
 }  // namespace
 
+bool gemv_takes_swiglu(WeightKind kind, int K) {
+    return (kind == WK_I8 || kind == WK_F16) && (K == 576 || K == 896 || K == 1024 || K == 1536);
+}
+
+// The kernels that keep x in registers, with 4-element virtual lanes.
+bool gemv_takes_norm(WeightKind kind, int K) {
+    return (kind == WK_I8 || kind == WK_F16) && (K == 576 || K == 896 || K == 1024 || K == 1536 || K == 4864);
+}
+
 bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
     if (n < 1 || n > kMaxSegments) {
         MI_ERROR_FMT("gemv: %d segments in one launch (1..%d allowed)", n, kMaxSegments);
@@ -798,14 +914,32 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
     for (int i = 0; i < n; ++i) {
         if (!check_call(calls[i])) return false;
         if (calls[i].x != calls[0].x || calls[i].K != calls[0].K || calls[i].kind != calls[0].kind ||
-            calls[i].M != calls[0].M || calls[i].epi != calls[0].epi) {
-            MI_ERROR_FMT("gemv: segments of one launch must share x, K, M, weight kind and epilogue");
+            calls[i].M != calls[0].M || calls[i].epi != calls[0].epi || calls[i].norm_w != calls[0].norm_w ||
+            calls[i].norm_eps != calls[0].norm_eps || calls[i].add_rounded != calls[0].add_rounded) {
+            MI_ERROR_FMT("gemv: segments of one launch must share x, K, M, weight kind, epilogue and norm");
             return false;
         }
         rows += calls[i].N;
     }
     const GemvCall& c = calls[0];
+    if (c.norm_w && !(gemv_takes_norm(c.kind, c.K) && aligned(c.norm_w, 16))) {
+        MI_ERROR_FMT("gemv: no fused RMSNorm for kind=%d K=%d (or misaligned norm weights)", static_cast<int>(c.kind), c.K);
+        return false;
+    }
     const int vl = pick_vl(c.kind, c.M, rows, c.K);
+    if (c.epi == EPI_SWIGLU) {
+        if (n != 2 || calls[0].N != calls[1].N || c.M != 1 || !gemv_takes_swiglu(c.kind, c.K)) {
+            MI_ERROR_FMT("gemv: the SwiGLU epilogue takes a gate and an up matrix of equal N, M = 1, int8 or fp16 "
+                         "weights and K in {576, 896, 1024, 1536} (n=%d kind=%d K=%d)", n, static_cast<int>(c.kind), c.K);
+            return false;
+        }
+        if (c.kind == WK_I8) {
+            if (vl == 4) return launch_swiglu_vl<WK_I8, 4>(s, calls);
+            if (vl == 2) return launch_swiglu_vl<WK_I8, 2>(s, calls);
+            return launch_swiglu_vl<WK_I8, 1>(s, calls);
+        }
+        return vl == 2 ? launch_swiglu_vl<WK_F16, 2>(s, calls) : launch_swiglu_vl<WK_F16, 1>(s, calls);
+    }
     const bool add = c.epi == EPI_ADD;
     if (c.kind == WK_Q4 && vl == 4 && gemv_mode() == 1) {
         bool taken = false;

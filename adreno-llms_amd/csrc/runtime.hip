@@ -81,6 +81,30 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 }  // namespace
 
 const DeviceInfo& device_info() { return g_dev; }
+
+bool fused_gemv_kind(const void* W, int N, int K, WeightKind* kind) {
+    Entry e;
+    if (!resolve("decode step", W, N, K, &e)) return false;
+    *kind = e.kind;
+    return true;
+}
+
+bool fused_gemv(hipStream_t s, int n, const int* N, int K, const void* x, const void* const* W, void* const* y,
+                const void* norm_w, float norm_eps, Epilogue epi) {
+    GemvCall group[kMaxSegments];
+    if (n < 1 || n > kMaxSegments) return false;
+    for (int i = 0; i < n; ++i) {
+        Entry e;
+        if (!resolve("decode step", W[i], N[i], K, &e)) return false;
+        GemvCall& d = group[i];
+        d.x = x; d.W = W[i]; d.scale = e.scale; d.y = y[i];
+        d.M = 1; d.N = N[i]; d.K = K; d.kind = e.kind;
+        d.epi = epi;
+        d.norm_w = norm_w; d.norm_eps = norm_eps; d.add_rounded = epi == EPI_ADD;
+    }
+    return launch_gemv_group(s, group, n);
+}
+
 int gemv_mode() { return g_gemv_mode; }
 int gemm_mode() { return g_gemm_mode; }
 

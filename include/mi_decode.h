@@ -68,6 +68,12 @@ int   mi_decoder_step(void* decoder, void* stream);
 int   mi_decoder_read(void* decoder, void* stream, int* pos, int* token);
 /* fp16 [vocab] logits of the last step, in device memory. */
 const void* mi_decoder_logits(void* decoder);
+/* Activations left by the last step, fp16 in device memory, for comparing implementations buffer
+ * by buffer: which = 0 residual stream [hidden], 1 q after bias and rotary [n_heads*head_dim],
+ * 2 k, 3 v [n_kv_heads*head_dim], 4 attention output [n_heads*head_dim], 5 swiglu(gate, up)
+ * [intermediate], all of the last layer; 6 / 7 the rotary cos / sin tables [max_pos*head_dim].
+ * NULL for any other value. */
+const void* mi_decoder_buffer(void* decoder, int which);
 
 #ifdef __cplusplus
 }

@@ -273,3 +273,22 @@ int orc_decoder_step(void* p, int token, int pos, orc_linear_fn fn, void* ctx, f
 }
 
 const uint16_t* orc_decoder_logits(void* p) { return ((orc_decoder*)p)->logits; }
+
+/* Activations left by the last step: 0 = residual stream h, 1 = q (after bias and rotary, last
+ * layer), 2 = k, 3 = v, 4 = attention output, 5 = swiglu(gate, up), 6 / 7 = the rotary cos / sin
+ * tables [max_pos][head_dim]; for comparing a device implementation buffer by buffer. */
+const uint16_t* orc_decoder_buffer(void* p, int which)
+{
+    orc_decoder* d = (orc_decoder*)p;
+    switch (which) {
+        case 0: return d->h;
+        case 1: return d->q;
+        case 2: return d->k;
+        case 3: return d->v;
+        case 4: return d->attn;
+        case 5: return d->gate;
+        case 6: return d->cosT;
+        case 7: return d->sinT;
+        default: return NULL;
+    }
+}

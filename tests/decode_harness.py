@@ -12,6 +12,9 @@ QWEN25_05B = dict(hidden=896, inter=4864, n_heads=14, n_kv_heads=2, head_dim=64,
                   vocab=151936, max_pos=64, rms_eps=1e-6, rope_theta=1000000.0)
 TINY = dict(hidden=64, inter=128, n_heads=4, n_kv_heads=2, head_dim=16, n_layers=2,
             vocab=512, max_pos=48, rms_eps=1e-6, rope_theta=10000.0)
+# SmolLM2-135M widths, cut to 3 layers and a small vocabulary: K = 576 and 1536
+SMOL = dict(hidden=576, inter=1536, n_heads=9, n_kv_heads=3, head_dim=64, n_layers=3,
+            vocab=4096, max_pos=48, rms_eps=1e-5, rope_theta=100000.0)
 PROMPT = [785, 11079, 6439, 518, 279, 220]       # QW/reference/test_input_ids.bin
 
 _PP16 = C.POINTER(C.POINTER(C.c_uint16))
@@ -33,6 +36,8 @@ _lib = O.lib
 _lib.orc_decoder_new.restype = C.c_void_p
 _lib.orc_decoder_new.argtypes = [C.POINTER(OrcModel), C.c_int]
 _lib.orc_decoder_free.argtypes = [C.c_void_p]
+_lib.orc_decoder_logits.restype = C.c_void_p
+_lib.orc_decoder_logits.argtypes = [C.c_void_p]
 _lib.orc_decoder_step.restype = C.c_int
 _lib.orc_decoder_step.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
 
@@ -91,9 +96,11 @@ class Model:
         return m
 
 
-def greedy(model, prompt, n_new, linear_cb=None, threads=O.THREADS):
+def greedy(model, prompt, n_new, linear_cb=None, threads=O.THREADS, last_logits=None):
     """Feeds the prompt token by token, then decodes n_new tokens greedily.
-    Returns (tokens, margins); linear_cb(index, x_ptr, y_ptr) replaces the oracle GEMV."""
+    Returns (tokens, margins); linear_cb(index, x_ptr, y_ptr) replaces the oracle GEMV.
+    last_logits: a uint16 array of vocab entries that receives the logits of the last step
+    that produced a listed token."""
     cs = model.c_struct()
     dec = _lib.orc_decoder_new(C.byref(cs), threads)
     fn = LINEAR_FN(lambda ctx, idx, x, y: linear_cb(idx, x, y)) if linear_cb else None
@@ -104,9 +111,14 @@ def greedy(model, prompt, n_new, linear_cb=None, threads=O.THREADS):
         for t in prompt:
             nxt = _lib.orc_decoder_step(dec, int(t) % model.cfg["vocab"], pos, fn_ptr, None, C.byref(margin))
             pos += 1
-        for _ in range(n_new):
+        for i in range(n_new):
             toks.append(nxt)
             margins.append(margin.value)
+            if i == n_new - 1:
+                if last_logits is not None:
+                    src = (C.c_uint16 * model.cfg["vocab"]).from_address(_lib.orc_decoder_logits(dec))
+                    last_logits[:] = np.ctypeslib.as_array(src)
+                break
             nxt = _lib.orc_decoder_step(dec, nxt, pos, fn_ptr, None, C.byref(margin))
             pos += 1
     finally:
@@ -181,6 +193,15 @@ class GpuDecoder:
             run()
             toks.append(d.read(q)[1])
         return toks
+
+    def logits(self):
+        """Logits of the last step, as stored by the lm_head (uint16 bit patterns)."""
+        vocab = self.model.cfg["vocab"]
+        out = np.empty(vocab, np.uint16)
+        self.queue.finish()
+        assert mil.lib().mi_memcpy_d2h(out.ctypes.data, self.dec.logits_ptr, vocab * 2, self.queue.handle)
+        self.queue.finish()
+        return out
 
     def close(self):
         self.dec.close()
