@@ -110,72 +110,93 @@ __global__ __launch_bounds__(64) void rmsnorm_kernel(const uint16_t* __restrict_
     for (int c = c4n * 4 + lid; c < cols; c += 64) out[c] = f_h((h_f(x[c]) * inv) * h_f(w[c]));
 }
 
-// q/k/v bias (QW/kernels/bias_add.cl), rotary embedding of q and k at the current position
-// (QW/kernels/rope.cl), then k and v into the caches (rows as QW/src/layers/attention.cpp:560-600):
-// one launch, each value rounded to fp16 where the separate kernels would store it.
-__global__ void bias_rope_kv_kernel(uint16_t* __restrict__ q, uint16_t* __restrict__ k, uint16_t* __restrict__ v,
-                                    const uint16_t* __restrict__ bq, const uint16_t* __restrict__ bk,
-                                    const uint16_t* __restrict__ bv, const uint16_t* __restrict__ cosT,
-                                    const uint16_t* __restrict__ sinT, uint16_t* __restrict__ kc,
-                                    uint16_t* __restrict__ vc, const State* __restrict__ st, int n_heads,
-                                    int n_kv_heads, int D, int max_pos) {
-    int pos = st->pos;
-    pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
-    const int hd2 = D / 2, kvd = n_kv_heads * D;
-    const uint16_t* cr = cosT + static_cast<size_t>(pos) * D;
-    const uint16_t* sr = sinT + static_cast<size_t>(pos) * D;
-    const int pairs = (n_heads + n_kv_heads) * hd2;
-    for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < pairs; p += gridDim.x * blockDim.x) {
-        const int head = p / hd2, i = p % hd2;
-        uint16_t* buf = head < n_heads ? q + head * D : k + (head - n_heads) * D;
-        const uint16_t* bias = head < n_heads ? bq + head * D : bk + (head - n_heads) * D;
-        const float x1 = h_f(f_h(h_f(buf[i]) + h_f(bias[i])));
-        const float x2 = h_f(f_h(h_f(buf[i + hd2]) + h_f(bias[i + hd2])));
-        const float c = h_f(cr[i]), s = h_f(sr[i]);
-        const float o1 = fmaf(x1, c, -(x2 * s));
-        const float o2 = fmaf(x2, c, x1 * s);
-        const uint16_t r1 = f_h(o1), r2 = f_h(o2);
-        buf[i] = r1;
-        buf[i + hd2] = r2;
-        if (head >= n_heads) {
-            uint16_t* dst = kc + static_cast<size_t>(pos) * kvd + (head - n_heads) * D;
-            dst[i] = r1;
-            dst[i + hd2] = r2;
-        }
-    }
-    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < kvd; e += gridDim.x * blockDim.x) {
-        const uint16_t r = f_h(h_f(v[e]) + h_f(bv[e]));
-        v[e] = r;
-        vc[static_cast<size_t>(pos) * kvd + e] = r;
-    }
-}
-
-// Single-query grouped-query attention for one head per block (QW/kernels/attention.cl:
-// gqa_attn_scores, gqa_softmax, gqa_attn_out).  Sums run in the order the CPU restatement uses:
-// the score over D in float4 groups, the softmax denominator over the keys in index order, the
-// output over the keys in index order.  The scores (fp16, as the reference's score buffer holds
-// them) and the fp32 exponentials stay in LDS: dynamic LDS of 6 bytes per position.
-__global__ void attention_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc,
-                                 const uint16_t* __restrict__ vc, uint16_t* __restrict__ out,
-                                 const State* __restrict__ st, int n_heads, int n_kv_heads, int D, int max_pos,
-                                 float scale) {
-    extern __shared__ float ex[];
-    uint16_t* sc = reinterpret_cast<uint16_t*>(ex + max_pos);
+// One block per query head: q/k/v bias (QW/kernels/bias_add.cl), rotary embedding of q and k at the
+// current position (QW/kernels/rope.cl), k and v into the caches (rows as QW/src/layers/
+// attention.cpp:560-600), then single-query grouped-query attention (QW/kernels/attention.cl:
+// gqa_attn_scores, gqa_softmax, gqa_attn_out); each value rounded to fp16 where the separate
+// kernels would store it.  Sums run in the order the CPU restatement uses: the score over D in
+// float4 groups, the softmax denominator over the keys in index order, the output over the keys
+// in index order.
+// Every head of a group prepares the group's k and v of the current position for itself (in
+// LDS; the values are the same in all of them) and reads only older rows from the caches; the
+// group's first head writes the new row.  raw = the projections' outputs; q_out, k_out, v_out
+// receive them after bias and rotary embedding.
+// Dynamic LDS: 6 bytes per position (fp32 exponentials, fp16 scores) + 6 D bytes.
+__global__ __launch_bounds__(256) void rope_attention_kernel(const uint16_t* __restrict__ q_raw, const uint16_t* __restrict__ k_raw,
+                                      const uint16_t* __restrict__ v_raw, const uint16_t* __restrict__ bq,
+                                      const uint16_t* __restrict__ bk, const uint16_t* __restrict__ bv,
+                                      const uint16_t* __restrict__ cosT, const uint16_t* __restrict__ sinT,
+                                      uint16_t* __restrict__ kc, uint16_t* __restrict__ vc,
+                                      uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_out,
+                                      uint16_t* __restrict__ v_out, uint16_t* __restrict__ out,
+                                      const State* __restrict__ st, int n_heads, int n_kv_heads, int D, int max_pos,
+                                      float scale) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t qv[];          // q, then k and v of the current position:
+    uint16_t* kcur = qv + D;                                               // 3 D halves (a multiple of 8 bytes)
+    uint16_t* vcur = kcur + D;
+    float* ex = reinterpret_cast<float*>(vcur + D);                        // [max_pos] exponentials
+    uint16_t* sc = reinterpret_cast<uint16_t*>(ex + max_pos);              // [max_pos] scores
     __shared__ float red[64];
     __shared__ float inv_s;
     int pos = st->pos;
     pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
-    const int seq_k = pos + 1, qh = blockIdx.x, kvd = n_kv_heads * D, kvh = qh / (n_heads / n_kv_heads);
+    const int nrep = n_heads / n_kv_heads;
+    const int seq_k = pos + 1, qh = blockIdx.x, kvd = n_kv_heads * D, kvh = qh / nrep, hd2 = D / 2;
+    const bool writer = qh % nrep == 0;
     const int tid = threadIdx.x, nt = blockDim.x;
-    const uint16_t* qv = q + qh * D;
+    const uint16_t* cr = cosT + static_cast<size_t>(pos) * D;
+    const uint16_t* sr = sinT + static_cast<size_t>(pos) * D;
+    for (int i = tid; i < hd2; i += nt) {
+        const float c = h_f(cr[i]), sn = h_f(sr[i]);
+        {
+            const uint16_t* buf = q_raw + qh * D;
+            const uint16_t* bias = bq + qh * D;
+            const float x1 = h_f(f_h(h_f(buf[i]) + h_f(bias[i])));
+            const float x2 = h_f(f_h(h_f(buf[i + hd2]) + h_f(bias[i + hd2])));
+            const uint16_t r1 = f_h(fmaf(x1, c, -(x2 * sn))), r2 = f_h(fmaf(x2, c, x1 * sn));
+            qv[i] = r1;
+            qv[i + hd2] = r2;
+            q_out[qh * D + i] = r1;
+            q_out[qh * D + i + hd2] = r2;
+        }
+        {
+            const uint16_t* buf = k_raw + kvh * D;
+            const uint16_t* bias = bk + kvh * D;
+            const float x1 = h_f(f_h(h_f(buf[i]) + h_f(bias[i])));
+            const float x2 = h_f(f_h(h_f(buf[i + hd2]) + h_f(bias[i + hd2])));
+            const uint16_t r1 = f_h(fmaf(x1, c, -(x2 * sn))), r2 = f_h(fmaf(x2, c, x1 * sn));
+            kcur[i] = r1;
+            kcur[i + hd2] = r2;
+            if (writer) {
+                uint16_t* dst = kc + static_cast<size_t>(pos) * kvd + kvh * D;
+                dst[i] = r1;
+                dst[i + hd2] = r2;
+                k_out[kvh * D + i] = r1;
+                k_out[kvh * D + i + hd2] = r2;
+            }
+        }
+    }
+    for (int e = tid; e < D; e += nt) {
+        const uint16_t r = f_h(h_f(v_raw[kvh * D + e]) + h_f(bv[kvh * D + e]));
+        vcur[e] = r;
+        if (writer) {
+            vc[static_cast<size_t>(pos) * kvd + kvh * D + e] = r;
+            v_out[kvh * D + e] = r;
+        }
+    }
+    __syncthreads();
     for (int tk = tid; tk < seq_k; tk += nt) {
-        const uint16_t* kv = kc + static_cast<size_t>(tk) * kvd + kvh * D;
+        // a key row is read in 8-byte pieces (rows start at multiples of 8 bytes: D % 4 == 0)
+        typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+        const u16x4* kv = reinterpret_cast<const u16x4*>(tk == pos ? kcur : kc + static_cast<size_t>(tk) * kvd + kvh * D);
+        const u16x4* qq = reinterpret_cast<const u16x4*>(qv);
         float acc = 0.0f;
         for (int d4 = 0; d4 < D / 4; ++d4) {
-            float t = h_f(qv[4 * d4]) * h_f(kv[4 * d4]);
-            t = fmaf(h_f(qv[4 * d4 + 1]), h_f(kv[4 * d4 + 1]), t);
-            t = fmaf(h_f(qv[4 * d4 + 2]), h_f(kv[4 * d4 + 2]), t);
-            t = fmaf(h_f(qv[4 * d4 + 3]), h_f(kv[4 * d4 + 3]), t);
+            const u16x4 a = qq[d4], b = kv[d4];
+            float t = h_f(a[0]) * h_f(b[0]);
+            t = fmaf(h_f(a[1]), h_f(b[1]), t);
+            t = fmaf(h_f(a[2]), h_f(b[2]), t);
+            t = fmaf(h_f(a[3]), h_f(b[3]), t);
             acc = acc + t;
         }
         sc[tk] = f_h(acc * scale);
@@ -207,9 +228,19 @@ __global__ void attention_kernel(const uint16_t* __restrict__ q, const uint16_t*
     for (int c = tid; c < seq_k; c += nt) sc[c] = f_h(h_f(sc[c]) * inv);
     __syncthreads();
     for (int e = tid; e < D; e += nt) {
+        // keys 0 .. pos - 1 from the cache, eight loads in flight at a time, then the current one
+        const uint16_t* col = vc + kvh * D + e;
         float acc = 0.0f;
-        for (int tk = 0; tk < seq_k; ++tk)
-            acc = fmaf(h_f(sc[tk]), h_f(vc[static_cast<size_t>(tk) * kvd + kvh * D + e]), acc);
+        int tk = 0;
+        for (; tk + 8 <= pos; tk += 8) {
+            uint16_t v[8];
+            #pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = col[static_cast<size_t>(tk + u) * kvd];
+            #pragma unroll
+            for (int u = 0; u < 8; ++u) acc = fmaf(h_f(sc[tk + u]), h_f(v[u]), acc);
+        }
+        for (; tk < pos; ++tk) acc = fmaf(h_f(sc[tk]), h_f(col[static_cast<size_t>(tk) * kvd]), acc);
+        acc = fmaf(h_f(sc[pos]), h_f(vcur[e]), acc);
         out[qh * D + e] = f_h(acc);
     }
 }
@@ -237,6 +268,7 @@ struct Decoder {
     // device memory owned by the decoder
     uint16_t *kc = nullptr, *vc = nullptr, *cosT = nullptr, *sinT = nullptr;
     uint16_t *h = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr;
+    uint16_t *qr = nullptr, *kr = nullptr, *vr = nullptr;      // q, k, v after bias and rotary embedding
     uint16_t *gate = nullptr, *up = nullptr, *logits = nullptr;
     State* st = nullptr;
     std::vector<void*> owned;
@@ -264,7 +296,7 @@ void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* 
     if (!cfg || !w || mi_init(0) != 1) return nullptr;
     const mi_decoder_config& c = *cfg;
     if (c.hidden <= 0 || c.inter <= 0 || c.n_heads <= 0 || c.n_kv_heads <= 0 || c.head_dim <= 0 || c.n_layers <= 0 ||
-        c.vocab <= 0 || c.max_pos <= 0 || c.n_heads % c.n_kv_heads || c.head_dim % 4 || c.max_pos > 8192) {
+        c.vocab <= 0 || c.max_pos <= 0 || c.n_heads % c.n_kv_heads || c.head_dim % 4 || c.head_dim > 256 || c.max_pos > 8192) {
         MI_ERROR_FMT("mi_decoder_create: bad configuration");
         return nullptr;
     }
@@ -295,7 +327,8 @@ void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* 
               dev_alloc(d, &d->cosT, static_cast<size_t>(c.max_pos) * D * 2) &&
               dev_alloc(d, &d->sinT, static_cast<size_t>(c.max_pos) * D * 2) &&
               dev_alloc(d, &d->h, c.hidden * 2) && dev_alloc(d, &d->xn, c.hidden * 2) && dev_alloc(d, &d->q, qd * 2) &&
-              dev_alloc(d, &d->k, kvd * 2) && dev_alloc(d, &d->v, kvd * 2) && dev_alloc(d, &d->attn, qd * 2) &&
+              dev_alloc(d, &d->k, kvd * 2) && dev_alloc(d, &d->v, kvd * 2) && dev_alloc(d, &d->qr, qd * 2) &&
+              dev_alloc(d, &d->kr, kvd * 2) && dev_alloc(d, &d->vr, kvd * 2) && dev_alloc(d, &d->attn, qd * 2) &&
               dev_alloc(d, &d->gate, c.inter * 2) &&
               dev_alloc(d, &d->up, c.inter * 2) && dev_alloc(d, &d->logits, static_cast<size_t>(c.vocab) * 2) &&
               dev_alloc(d, &d->st, sizeof(State));
@@ -373,9 +406,9 @@ const void* mi_decoder_buffer(void* dec, int which) {
     if (!d) return nullptr;
     switch (which) {
         case 0: return d->h;
-        case 1: return d->q;
-        case 2: return d->k;
-        case 3: return d->v;
+        case 1: return d->qr;
+        case 2: return d->kr;
+        case 3: return d->vr;
         case 4: return d->attn;
         case 5: return d->gate;
         case 6: return d->cosT;
@@ -442,15 +475,11 @@ int mi_decoder_step(void* dec, void* stream) {
         }
         uint16_t* kc = d->kc + static_cast<size_t>(l) * c.max_pos * kvd;
         uint16_t* vc = d->vc + static_cast<size_t>(l) * c.max_pos * kvd;
-        const int pairs = (c.n_heads + c.n_kv_heads) * D / 2;
-        hipLaunchKernelGGL(bias_rope_kv_kernel, dim3((pairs + 255) / 256), dim3(256), 0, s, d->q, d->k, d->v,
-                           static_cast<const uint16_t*>(d->bq[l]), static_cast<const uint16_t*>(d->bk[l]),
-                           static_cast<const uint16_t*>(d->bv[l]), d->cosT, d->sinT, kc, vc, d->st, c.n_heads,
-                           c.n_kv_heads, D, c.max_pos);
-        if (!launched()) return 0;
         const int at = D > 64 ? D : 64;
-        hipLaunchKernelGGL(attention_kernel, dim3(c.n_heads), dim3(at), static_cast<size_t>(c.max_pos) * 6, s, d->q, kc, vc,
-                           d->attn, d->st, c.n_heads, c.n_kv_heads, D, c.max_pos, scale);
+        hipLaunchKernelGGL(rope_attention_kernel, dim3(c.n_heads), dim3(at), static_cast<size_t>(c.max_pos) * 6 + D * 6, s,
+                           d->q, d->k, d->v, static_cast<const uint16_t*>(d->bq[l]), static_cast<const uint16_t*>(d->bk[l]),
+                           static_cast<const uint16_t*>(d->bv[l]), d->cosT, d->sinT, kc, vc, d->qr, d->kr, d->vr, d->attn,
+                           d->st, c.n_heads, c.n_kv_heads, D, c.max_pos, scale);
         if (!launched()) return 0;
         if (!linear_into_h(qd, d->attn, d->wo[l])) return 0;
         {

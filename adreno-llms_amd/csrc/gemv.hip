@@ -926,7 +926,9 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
         MI_ERROR_FMT("gemv: no fused RMSNorm for kind=%d K=%d (or misaligned norm weights)", static_cast<int>(c.kind), c.K);
         return false;
     }
-    const int vl = pick_vl(c.kind, c.M, rows, c.K);
+    // (SwiGLU: a wavefront takes a row batch of both matrices, so there are half as many
+    //  wavefronts as batches; the lane tile is picked for that count)
+    const int vl = pick_vl(c.kind, c.M, c.epi == EPI_SWIGLU ? rows / 4 : rows, c.K);
     if (c.epi == EPI_SWIGLU) {
         if (n != 2 || calls[0].N != calls[1].N || c.M != 1 || !gemv_takes_swiglu(c.kind, c.K)) {
             MI_ERROR_FMT("gemv: the SwiGLU epilogue takes a gate and an up matrix of equal N, M = 1, int8 or fp16 "
