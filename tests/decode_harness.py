@@ -126,6 +126,37 @@ def greedy(model, prompt, n_new, linear_cb=None, threads=O.THREADS, last_logits=
     return toks, margins
 
 
+class KindModel(Model):
+    """The same model with every projection stored as fp16 ("f16") or block-32 Q4 ("q4") instead of
+    int8: the CPU harness reaches the matching oracle GEMV through the callback, the device decoder
+    gets the weights registered (or not, for fp16) accordingly."""
+
+    def __init__(self, cfg, kind, seed=2024):
+        super().__init__(cfg, seed)
+        assert kind in ("f16", "q4")
+        self.kind = kind
+        s = seed * 1000
+        self.wf, self.wq4 = [], []
+        for i, (N, K) in enumerate(self.shapes):
+            w = mil.synth_normal_f16(s + 1 + (i if i < len(self.shapes) - 1 else 399), 0.02, (N, K))
+            if kind == "f16":
+                self.wf.append(w)
+            else:
+                self.wq4.append(mil.quantize_q4(w))
+
+    def oracle_cb(self):
+        def cb(idx, x_ptr, y_ptr):
+            N, K = self.shapes[idx]
+            x = np.ctypeslib.as_array((C.c_uint16 * K).from_address(x_ptr))
+            y = np.ctypeslib.as_array((C.c_uint16 * N).from_address(y_ptr))
+            if self.kind == "f16":
+                y[:] = O.gemv_f16(x.view(np.float16), self.wf[idx])
+            else:
+                p, sc = self.wq4[idx]
+                y[:] = O.gemv_q4(x.view(np.float16), p, sc.view(np.uint16))
+        return cb
+
+
 class GpuLinear:
     """The library behind the callback: weights resident and registered once, x up, y down."""
 
@@ -160,10 +191,19 @@ class GpuDecoder:
     def __init__(self, model, queue):
         c = model.cfg
         self.model, self.queue = model, queue
-        self.W = [mil.Buffer.from_host(q) for q in model.w8]
-        self.S = [mil.Buffer.from_host(s) for s in model.ws]
-        for (N, K), w, s in zip(model.shapes, self.W, self.S):
-            assert mil.nnopt_register_int8_weight(w, s, N, K)
+        kind = getattr(model, "kind", "i8")
+        if kind == "f16":
+            self.W, self.S = [mil.Buffer.from_host(w) for w in model.wf], []
+        elif kind == "q4":
+            self.W = [mil.Buffer.from_host(p) for p, _ in model.wq4]
+            self.S = [mil.Buffer.from_host(sc) for _, sc in model.wq4]
+            for (N, K), w, s in zip(model.shapes, self.W, self.S):
+                assert mil.nnopt_register_q4_weight(w, s, N, K)
+        else:
+            self.W = [mil.Buffer.from_host(q) for q in model.w8]
+            self.S = [mil.Buffer.from_host(s) for s in model.ws]
+            for (N, K), w, s in zip(model.shapes, self.W, self.S):
+                assert mil.nnopt_register_int8_weight(w, s, N, K)
         up = lambda arrs: [mil.Buffer.from_host(a) for a in arrs]
         L = c["n_layers"]
         self.bufs = dict(embed=mil.Buffer.from_host(model.embed), final_norm=mil.Buffer.from_host(model.final_norm),

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as O
-from decode_harness import PROMPT, QWEN25_05B, SMOL, TINY, GpuDecoder, GpuLinear, Model, greedy
+from decode_harness import PROMPT, QWEN25_05B, SMOL, TINY, GpuDecoder, GpuLinear, KindModel, Model, greedy
 from helpers import mil
 
 
@@ -120,6 +120,30 @@ def test_qwen_shaped_whole_step_on_device_graph_replay():
     assert got == want
     assert np.array_equal(got_logits, want_logits)      # every bit of the last step's 151936 logits
     assert pos == len(PROMPT) - 1 + 32       # the first prompt token is set by reset, every later token costs a step
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["f16", "q4"])
+def test_smollm_widths_fp16_and_q4_weights_on_device(kind):
+    """The device step with fp16 weights (norm, add and SwiGLU ride in the fp16 GEMV kernels) and with
+    Q4 weights (no fused norm for 8-element lanes: separate norm and SwiGLU launches, add in the
+    epilogue), exact GEMV mode: tokens and last logits equal the CPU harness running the oracle's
+    GEMV of the same kind."""
+    assert mil.lib().mi_init(0) == 1
+    mil.lib().mi_set_gemv_mode(0)
+    try:
+        queue = mil.Queue()
+        m = KindModel(SMOL, kind, seed=9)
+        want_logits = np.empty(SMOL["vocab"], np.uint16)
+        want, _ = greedy(m, PROMPT, 24, linear_cb=m.oracle_cb(), last_logits=want_logits)
+        gd = GpuDecoder(m, queue)
+        got = gd.greedy(PROMPT, 24)
+        got_logits = gd.logits()
+        gd.close()
+        assert got == want and len(set(got)) > 1
+        assert np.array_equal(got_logits, want_logits)
+    finally:
+        mil.lib().mi_set_gemv_mode(1)
 
 
 @pytest.mark.gpu
