@@ -52,6 +52,7 @@ _SIGNATURES = {
     "mi_graph_destroy": (_i, [_vp]),
     "mi_linear_add": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
     "mi_linear_gate_up_silu": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp]),
+    "mi_linear_silu_gate": (_i, [_vp, _i, _i, _vp, _vp, _vp]),
     "mi_dequant_int8_to_fp16": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "mi_unpack_q4_to_int8": (_i, [_vp, _vp, _i, _i, _vp]),
     "mi_decoder_create": (_vp, [_vp, _vp]),
@@ -253,6 +254,11 @@ def pytorch_linear_add(queue, M, N, K, x, W, residual_inout):
 def fused_gate_up_silu_m1(queue, N, K, x, Wg, Wu, out):
     """out = silu(Wg x) * (Wu x) (QW/src/utils.h:157-159).  False = not taken."""
     return bool(lib().mi_linear_gate_up_silu(_q(queue), N, K, _h(x), _h(Wg), _h(Wu), _h(out)))
+
+
+def pytorch_linear_silu_gate_fused(queue, N, K, x, W3, gate_inout):
+    """gate_inout = silu(gate_inout) * (W3 x) (LF/src/utils.h:140-142).  False = not taken."""
+    return bool(lib().mi_linear_silu_gate(_q(queue), N, K, _h(x), _h(W3), _h(gate_inout)))
 
 
 def nnopt_register_int8_weight(W_int8, scale_fp16, N, K):

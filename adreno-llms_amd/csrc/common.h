@@ -25,6 +25,10 @@ enum WeightKind : int { WK_F16 = 0, WK_Q4 = 4, WK_I8 = 8 };
 // EPI_SWIGLU: two segments, gate and up, of equal N: y_gate[n] = swiglu(fp16(gate row n), fp16(up row n)),
 // the unfused sequence of two GEMVs and the element-wise kernel; y_up is not written.
 enum Epilogue : int { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2 };
+// EPI_ADD combines the product with the value y holds: y = fp16(y + product) in one rounding
+// (ADD_FUSED), y = fp16(fp16(product) + y) as a GEMV followed by an element-wise add gives
+// (ADD_ROUNDED), or y = fp16((y * sigmoid(y)) * product), y being the gate of a SwiGLU (ADD_SILU_GATE).
+enum AddMode : int { ADD_FUSED = 0, ADD_ROUNDED = 1, ADD_SILU_GATE = 2 };
 
 struct DeviceInfo {
     int  device = -1;
@@ -49,7 +53,7 @@ struct GemvCall {
     // Decode-step fusions (no counterpart at the C boundary):
     const void* norm_w = nullptr; // fp16 [K]: x is RMS-normalised with these weights first (M = 1, see gemv_takes_norm)
     float       norm_eps = 0.0f;
-    bool        add_rounded = false;  // EPI_ADD: y = fp16(fp16(product) + y), the unfused GEMV-then-add sequence
+    int         add_mode = 0;         // EPI_ADD: an AddMode
 };
 
 // gemv.hip

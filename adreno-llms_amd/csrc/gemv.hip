@@ -58,13 +58,20 @@ struct SegList {
     int nbatch;      // row batches of all segments
     const uint16_t* norm_w;   // not null: x is RMS-normalised with these weights before use
     float norm_eps;
-    int add_rounded;          // EPI_ADD: the product is rounded to fp16 before the residual is added
+    int add_mode;             // EPI_ADD: an AddMode
 };
 
-// EPI_ADD, the two forms: the fused one of the reference's residual kernels (one rounding), and
-// the unfused sequence GEMV, then element-wise add of two fp16 vectors (two roundings).
-__device__ __forceinline__ float add_residual(float sum, float s, float res, bool scaled, int rounded) {
-    if (rounded) return h_f(f_h(scaled ? sum * s : sum)) + res;
+// EPI_ADD, what happens to the value y already holds (res):
+//  ADD_FUSED     the reference's residual kernels, one rounding: fp16(res + product)
+//  ADD_ROUNDED   the unfused sequence GEMV, then element-wise add of two fp16 vectors: two roundings
+//  ADD_SILU_GATE res is the gate of a SwiGLU: fp16((res * sigmoid(res)) * product)
+//                (LF/kernels/mlp_fused.cl:70-78: gate * sig * w3x on the fp32 product)
+__device__ __forceinline__ float add_residual(float sum, float s, float res, bool scaled, int mode) {
+    if (mode == ADD_ROUNDED) return h_f(f_h(scaled ? sum * s : sum)) + res;
+    if (mode == ADD_SILU_GATE) {
+        const float sig = __fdiv_rn(1.0f, 1.0f + exp_poly(-res));
+        return (res * sig) * (scaled ? sum * s : sum);
+    }
     return scaled ? fmaf(sum, s, res) : sum + res;
 }
 
@@ -382,9 +389,9 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
             float out;
             if constexpr (KIND == WK_I8) {
                 const float s = h_f(b.s[0]);
-                out = EPI == EPI_ADD ? add_residual(sum, s, h_f(b.res), true, L.add_rounded) : sum * s;
+                out = EPI == EPI_ADD ? add_residual(sum, s, h_f(b.res), true, L.add_mode) : sum * s;
             } else {
-                out = EPI == EPI_ADD ? add_residual(sum, 1.0f, h_f(b.res), false, L.add_rounded) : sum;
+                out = EPI == EPI_ADD ? add_residual(sum, 1.0f, h_f(b.res), false, L.add_mode) : sum;
             }
             b.ybase[b.yoff] = f_h(out);
         }
@@ -541,7 +548,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
         acc = add_from_above<2>(acc);
         acc = add_from_above<1>(acc);
         if (g == 0 && b.yoff >= 0) {
-            const float out = EPI == EPI_ADD ? add_residual(acc, 1.0f, h_f(b.res), false, L.add_rounded) : acc;
+            const float out = EPI == EPI_ADD ? add_residual(acc, 1.0f, h_f(b.res), false, L.add_mode) : acc;
             b.ybase[b.yoff] = f_h(out);
         }
     };
@@ -628,9 +635,9 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict_
             float out;
             if constexpr (KIND == WK_I8) {
                 const float s = h_f(sg.sc[row]);
-                out = EPI == EPI_ADD ? add_residual(sum, s, h_f(*yp), true, L.add_rounded) : sum * s;
+                out = EPI == EPI_ADD ? add_residual(sum, s, h_f(*yp), true, L.add_mode) : sum * s;
             } else {
-                out = EPI == EPI_ADD ? add_residual(sum, 1.0f, h_f(*yp), false, L.add_rounded) : sum;
+                out = EPI == EPI_ADD ? add_residual(sum, 1.0f, h_f(*yp), false, L.add_mode) : sum;
             }
             *yp = f_h(out);
         }
@@ -764,7 +771,7 @@ Plan make_plan(const GemvCall* calls, int n, int vl) {
     p.L.nbatch = first;
     p.L.norm_w = static_cast<const uint16_t*>(calls[0].norm_w);
     p.L.norm_eps = calls[0].norm_eps;
-    p.L.add_rounded = calls[0].add_rounded ? 1 : 0;
+    p.L.add_mode = calls[0].add_mode;
     const int cap = resident_waves();
     int waves = first;
     p.pipe = false;
@@ -915,7 +922,7 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
         if (!check_call(calls[i])) return false;
         if (calls[i].x != calls[0].x || calls[i].K != calls[0].K || calls[i].kind != calls[0].kind ||
             calls[i].M != calls[0].M || calls[i].epi != calls[0].epi || calls[i].norm_w != calls[0].norm_w ||
-            calls[i].norm_eps != calls[0].norm_eps || calls[i].add_rounded != calls[0].add_rounded) {
+            calls[i].norm_eps != calls[0].norm_eps || calls[i].add_mode != calls[0].add_mode) {
             MI_ERROR_FMT("gemv: segments of one launch must share x, K, M, weight kind, epilogue and norm");
             return false;
         }

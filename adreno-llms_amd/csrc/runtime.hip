@@ -100,7 +100,7 @@ bool fused_gemv(hipStream_t s, int n, const int* N, int K, const void* x, const 
         d.x = x; d.W = W[i]; d.scale = e.scale; d.y = y[i];
         d.M = 1; d.N = N[i]; d.K = K; d.kind = e.kind;
         d.epi = epi;
-        d.norm_w = norm_w; d.norm_eps = norm_eps; d.add_rounded = epi == EPI_ADD;
+        d.norm_w = norm_w; d.norm_eps = norm_eps; d.add_mode = epi == EPI_ADD ? ADD_ROUNDED : ADD_FUSED;
     }
     return launch_gemv_group(s, group, n);
 }
@@ -390,6 +390,20 @@ int mi_linear_add(void* stream, int M, int N, int K, const void* x, const void* 
     GemvCall c;
     c.x = x; c.W = W; c.scale = e.scale; c.y = residual;
     c.M = 1; c.N = N; c.K = K; c.kind = e.kind; c.epi = EPI_ADD;
+    return launch_gemv(as_stream(stream), c) ? 1 : 0;
+}
+
+int mi_linear_silu_gate(void* stream, int N, int K, const void* x, const void* W, void* gate_inout) {
+    if (!ensure_init()) return 0;
+    if (N <= 0 || K <= 0 || !x || !W || !gate_inout) {
+        MI_ERROR_FMT("mi_linear_silu_gate: bad argument (N=%d K=%d)", N, K);
+        return 0;
+    }
+    Entry e;
+    if (!resolve("mi_linear_silu_gate", W, N, K, &e)) return 0;
+    GemvCall c;
+    c.x = x; c.W = W; c.scale = e.scale; c.y = gate_inout;
+    c.M = 1; c.N = N; c.K = K; c.kind = e.kind; c.epi = EPI_ADD; c.add_mode = ADD_SILU_GATE;
     return launch_gemv(as_stream(stream), c) ? 1 : 0;
 }
 

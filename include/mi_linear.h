@@ -90,6 +90,14 @@ int mi_linear_add(void* stream, int M, int N, int K, const void* x, const void* 
  * must be of the same kind (both fp16 or both int8); returns 0 otherwise. */
 int mi_linear_gate_up_silu(void* stream, int N, int K, const void* x, const void* Wg, const void* Wu, void* out);
 
+/* pytorch_linear_silu_gate_fused (LF/src/utils.h:140-142, LF/src/utils.cpp:1377-1406; kernel
+ * LF/kernels/mlp_fused.cl:19-79): the second projection of a SwiGLU with the activation behind it.
+ * gate_inout[n] holds (W1 x)[n] from an earlier mi_linear call and becomes
+ * fp16((gate * sigmoid(gate)) * (W x)[n]), the product W x entering in fp32.  M = 1.  The reference
+ * takes fp16 weights at K = 1024 only and returns false otherwise; here every kind and K of
+ * mi_linear is taken (int8 and Q4: the scaled fp32 product). */
+int mi_linear_silu_gate(void* stream, int N, int K, const void* x, const void* W, void* gate_inout);
+
 /* dequant_int8_weight_to_fp16 (LV/src/utils.cpp:594-634, LV/kernels/lfm2_ops.cl:731-743):
  * w16[n,k] = fp16(f32(q[n,k]) * f32(scale[n])). */
 int mi_dequant_int8_to_fp16(void* stream, const void* W_int8, const void* scale_fp16, int N, int K, void* w16);

@@ -401,6 +401,41 @@ void orc_gate_up_silu_f16(const uint16_t* x, const uint16_t* Wg, const uint16_t*
     free(xf);
 }
 
+/* LF/kernels/mlp_fused.cl:19-79 (gemv_m1_k1024_no8_silufused_img): the fp32 row sum w3x, then
+ * gate[n] = fp16(gate * sig * w3x) with sig = 1 / (1 + exp(-gate)), gate read as fp16.  The
+ * reference has the fp16 form only; int8 and Q4 take the scaled row sum of their GEMV. */
+static inline float silu_gate(float gate, float w3x)
+{
+    float sig = 1.0f / (1.0f + orc_expf(-gate));
+    return (gate * sig) * w3x;
+}
+
+void orc_gemv_f16_silu_gate(const uint16_t* x, const uint16_t* W, uint16_t* gate, int N, int K)
+{
+    float* xf = x_to_f32(x, K);
+    for (int n = 0; n < N; ++n)
+        gate[n] = orc_f32_to_f16(silu_gate(orc_f16_to_f32(gate[n]), row_f16(xf, W + (size_t)n * K, K)));
+    free(xf);
+}
+
+void orc_gemv_i8_silu_gate(const uint16_t* x, const int8_t* q, const uint16_t* s, uint16_t* gate, int N, int K)
+{
+    float* xf = x_to_f32(x, K);
+    for (int n = 0; n < N; ++n)
+        gate[n] = orc_f32_to_f16(silu_gate(orc_f16_to_f32(gate[n]),
+                                           row_i8(xf, q + (size_t)n * K, K) * orc_f16_to_f32(s[n])));
+    free(xf);
+}
+
+void orc_gemv_q4_silu_gate(const uint16_t* x, const uint8_t* p, const uint16_t* sc, uint16_t* gate, int N, int K)
+{
+    float* xf = x_to_f32(x, K);
+    for (int n = 0; n < N; ++n)
+        gate[n] = orc_f32_to_f16(silu_gate(orc_f16_to_f32(gate[n]),
+                                           row_q4(xf, p + (size_t)n * (K / 2), sc + (size_t)n * (K / 32), K)));
+    free(xf);
+}
+
 /* ------------------------------------------------------------------- M > 1 */
 
 void orc_gemm_f16(const uint16_t* X, const uint16_t* W, uint16_t* out, int M, int N, int K, int nt)

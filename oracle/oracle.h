@@ -81,6 +81,12 @@ void orc_gate_up_silu_i8(const uint16_t* x, const int8_t* qg, const int8_t* qu,
 void orc_gate_up_silu_f16(const uint16_t* x, const uint16_t* Wg, const uint16_t* Wu,
                           uint16_t* out, int N, int K);
 
+/* LF/kernels/mlp_fused.cl:19-79: gate[n] = fp16((gate * sigmoid(gate)) * (W x)[n]), W x in fp32
+ * (the reference has the fp16 form; int8 and Q4 use the scaled row sum of their GEMV). */
+void orc_gemv_f16_silu_gate(const uint16_t* x, const uint16_t* W, uint16_t* gate, int N, int K);
+void orc_gemv_i8_silu_gate (const uint16_t* x, const int8_t* q, const uint16_t* s, uint16_t* gate, int N, int K);
+void orc_gemv_q4_silu_gate (const uint16_t* x, const uint8_t* p, const uint16_t* sc, uint16_t* gate, int N, int K);
+
 /* M > 1: out[M,N] row i = GEMV of X row i (LF/src/model.cpp:243-250). */
 void orc_gemm_f16(const uint16_t* X, const uint16_t* W, uint16_t* out, int M, int N, int K, int n_threads);
 void orc_gemm_i8 (const uint16_t* X, const int8_t* q, const uint16_t* s, uint16_t* out, int M, int N, int K, int n_threads);

@@ -40,6 +40,9 @@ def _load():
         "orc_gemv_f16_add": (None, [_u16p, _u16p, _u16p, I, I]),
         "orc_gemv_i8_add": (None, [_u16p, _i8p, _u16p, _u16p, I, I]),
         "orc_gemv_q4_add": (None, [_u16p, _u8p, _u16p, _u16p, I, I]),
+        "orc_gemv_f16_silu_gate": (None, [_u16p, _u16p, _u16p, I, I]),
+        "orc_gemv_i8_silu_gate": (None, [_u16p, _i8p, _u16p, _u16p, I, I]),
+        "orc_gemv_q4_silu_gate": (None, [_u16p, _u8p, _u16p, _u16p, I, I]),
         "orc_gate_up_silu_i8": (None, [_u16p, _i8p, _i8p, _u16p, _u16p, _u16p, I, I]),
         "orc_gate_up_silu_f16": (None, [_u16p, _u16p, _u16p, _u16p, I, I]),
         "orc_gemm_f16": (None, [_u16p, _u16p, _u16p, I, I, I, I]),

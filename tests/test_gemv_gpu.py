@@ -185,6 +185,34 @@ def test_residual_add_epilogue(queue, kind, N, K):
     mil.nnopt_unregister_weight(Wb)
 
 
+@pytest.mark.parametrize("kind", ["i8", "q4", "f16"])
+@pytest.mark.parametrize("N,K", [(4608, 1024), (1536, 576), (4864, 896), (896, 4864), (30, 320)])
+def test_silu_gate_epilogue(queue, kind, N, K):
+    """pytorch_linear_silu_gate_fused: gate_inout = fp16(silu(gate_inout) * (W3 x)), bit for bit
+    against the oracle (LFM2's shape first: K = 1024, N = 4608)."""
+    W, x = synth_w(25, N, K), synth_x(26, K)
+    gate0 = synth_x(27, N)
+    xb, gb = mil.Buffer.from_host(x), mil.Buffer.from_host(gate0)
+    want = gate0.view(np.uint16).copy()
+    if kind == "i8":
+        q, s = mil.quantize_int8(W)
+        Wb, sb = mil.Buffer.from_host(q), mil.Buffer.from_host(s)
+        assert mil.nnopt_register_int8_weight(Wb, sb, N, K)
+        O.lib.orc_gemv_i8_silu_gate(O.u16(x), q, s.view(np.uint16), want, N, K)
+    elif kind == "q4":
+        p, sc = mil.quantize_q4(W)
+        Wb, sb = mil.Buffer.from_host(p), mil.Buffer.from_host(sc)
+        assert mil.nnopt_register_q4_weight(Wb, sb, N, K)
+        O.lib.orc_gemv_q4_silu_gate(O.u16(x), p, np.ascontiguousarray(sc.view(np.uint16)), want, N, K)
+    else:
+        Wb = mil.Buffer.from_host(W)
+        O.lib.orc_gemv_f16_silu_gate(O.u16(x), O.u16(W), want, N, K)
+    assert mil.pytorch_linear_silu_gate_fused(queue, N, K, xb, Wb, gb)
+    queue.finish()
+    assert np.array_equal(gb.read(np.uint16, (N,)), want)
+    mil.nnopt_unregister_weight(Wb)
+
+
 @pytest.mark.parametrize("kind", ["i8", "f16"])
 @pytest.mark.parametrize("N,K", [(1536, 576), (4864, 896), (50, 64)])
 def test_gate_up_silu_epilogue(queue, kind, N, K):

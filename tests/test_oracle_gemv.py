@@ -221,6 +221,50 @@ def test_fused_epilogues():
     assert np.all(np.abs(O.f16(out).astype(np.float64) - want) <= np.abs(want) * 2**-9 + 1e-5)
 
 
+def test_silu_gate_epilogue_closed_form():
+    """gate = fp16(silu(gate) * (W x)) against float64, for the three weight kinds; and the special
+    cases that pin the operand roles: gate = 0 gives 0 whatever W x is, a large gate passes W x
+    times gate through (sigmoid -> 1), W x = 0 gives 0."""
+    rng = np.random.default_rng(25)
+    N, K = 24, 1024
+    W, x = _rand(N, K, 26)
+    q, s = O.quantize_int8(W)
+    p, sc = O.quantize_q4(W)
+    gate0 = (rng.standard_normal(N) * 2).astype(np.float16)
+    xs = O.u16(x)
+    sig = lambda g: g / (1 + np.exp(-g))
+    x64, g64 = x.astype(np.float64), gate0.astype(np.float64)
+
+    gate = O.u16(gate0).copy()
+    O.lib.orc_gemv_f16_silu_gate(xs, O.u16(W), gate, N, K)
+    want = sig(g64) * (W.astype(np.float64) @ x64)
+    assert np.all(np.abs(O.f16(gate).astype(np.float64) - want) <= np.abs(want) * 2**-9 + 1e-5)
+
+    gate = O.u16(gate0).copy()
+    O.lib.orc_gemv_i8_silu_gate(xs, q, s, gate, N, K)
+    want = sig(g64) * ((q.astype(np.float64) @ x64) * O.f16(s))
+    assert np.all(np.abs(O.f16(gate).astype(np.float64) - want) <= np.abs(want) * 2**-9 + 1e-5)
+
+    gate = O.u16(gate0).copy()
+    O.lib.orc_gemv_q4_silu_gate(xs, p, np.ascontiguousarray(sc), gate, N, K)
+    wq4 = np.empty((N, K), np.float32)
+    O.lib.orc_dequant_q4_to_f32(p, np.ascontiguousarray(sc), N, K, wq4)
+    want = sig(g64) * (wq4.astype(np.float64) @ x64)
+    assert np.all(np.abs(O.f16(gate).astype(np.float64) - want) <= np.abs(want) * 2**-9 + 1e-5)
+
+    zero = np.zeros(N, np.uint16)
+    O.lib.orc_gemv_f16_silu_gate(xs, O.u16(W), zero, N, K)
+    assert not (zero & 0x7FFF).any()                            # silu(0) = 0 (of either sign)
+    big = O.u16(np.full(N, 30.0, np.float16)).copy()
+    O.lib.orc_gemv_f16_silu_gate(xs, O.u16(W), big, N, K)       # sigmoid(30) rounds to 1 in fp32
+    y = np.empty(N, np.float64)
+    want = (30.0 * (W.astype(np.float64) @ x64))
+    assert np.all(np.abs(O.f16(big).astype(np.float64) - want) <= np.abs(want) * 2**-10 + 1e-6)
+    gate = O.u16(gate0).copy()
+    O.lib.orc_gemv_f16_silu_gate(O.u16(np.zeros(K, np.float16)), O.u16(W), gate, N, K)
+    assert not (gate & 0x7FFF).any()                            # W x = 0
+
+
 def test_gemm_rows_are_gemvs():
     M, N, K = 5, 12, 896
     rng = np.random.default_rng(18)
