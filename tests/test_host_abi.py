@@ -45,3 +45,41 @@ def test_register_argument_checks_need_no_gpu(capfd):
     assert L.mi_unregister_weight(0x1000) == 1
     assert L.mi_weight_kind(0x1000) == 0
     assert L.mi_unregister_weight(0x1000) == 0
+
+
+def test_headers_are_plain_c_and_a_c_program_links(tmp_path):
+    """The boundary is a C ABI: both headers compile as C11 with gcc (no C++, no HIP types), and a C
+    program that calls the host-only entry points links against the library and runs without a GPU."""
+    import subprocess
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include "mi_linear.h"
+#include "mi_decode.h"
+#include <stdio.h>
+#include <string.h>
+int main(void) {
+    uint16_t w[2 * 32];
+    int8_t q[2 * 32];
+    uint8_t p[2 * 16];
+    uint16_t s8[2], s4[2];
+    mi_synth_normal_f16(7, 0.02, 2 * 32, w);
+    if (!mi_quantize_int8(w, 2, 32, q, s8)) return 1;
+    if (!mi_quantize_q4(w, 2, 32, p, s4)) return 2;
+    mi_linear_call call;
+    memset(&call, 0, sizeof call);
+    mi_decoder_config cfg;
+    memset(&cfg, 0, sizeof cfg);
+    if (mi_decoder_create(&cfg, 0) != 0) return 3;          /* refused: bad configuration, no device touched */
+    printf("ok %d %d\n", (int)q[0], (int)p[0]);
+    return 0;
+}
+''')
+    exe = tmp_path / "abi"
+    inc = os.path.join(ROOT, "include")
+    libdir = os.path.dirname(mil.LIB_PATH)
+    cmd = ["gcc", "-std=c11", "-Wall", "-Werror", "-pedantic", "-I", inc, str(src), "-o", str(exe),
+           "-L", libdir, "-lmi_linear", f"-Wl,-rpath,{libdir}"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0 and r.stdout.startswith("ok"), (r.returncode, r.stdout, r.stderr)
