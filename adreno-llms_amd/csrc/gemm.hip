@@ -193,22 +193,22 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const uint16_t* __restri
     }
 }
 
-// ---- int8 weights, wide tiles fed by direct global -> LDS loads ------------------------
+// ---- wide tiles fed by direct global -> LDS loads (int8, Q4 and fp16 weights) ----------
 //
 // What bounds the kernel above is the rate at which a CU can fill LDS (about 150 bytes/ns,
 // against 530 bytes/ns for reads and one 32x32x16 MFMA per 15.6 ns per SIMD) and the fragment
 // reads that are not overlapped with the MFMAs of the same wavefront.  This kernel therefore
-//  * keeps W as int8 in LDS (half the fill bytes) and converts a fragment to fp16 in registers
-//    after reading it; the four wavefronts of a block own disjoint rows of W (64 each, so the
-//    block covers 256 rows of W) and share the 32*TM rows of x, so no fragment of W is
-//    converted twice;
-//  * fills LDS with global_load_lds_dwordx4 (no registers, no ds_write), four to eight stages of K = 64;
-//    16-byte chunks are XOR-swizzled inside a row so that fragment reads are conflict-free
+//  * keeps quantised W as it is stored (int8, or Q4 nibbles with their block scales) in LDS
+//    (a half or a quarter of the fill bytes) and converts a fragment to fp16 in registers after
+//    reading it; the four wavefronts of a block own disjoint rows of W (64 each, so the block
+//    covers 256 rows of W) and share the 32*TM rows of x, so no fragment of W is converted twice;
+//  * fills LDS with global_load_lds_dwordx4 (no registers, no ds_write), three to eight stages of
+//    K = 64; 16-byte chunks are XOR-swizzled inside a row so that fragment reads are conflict-free
 //    without padding (a wavefront's load always fills 1 KB of consecutive LDS);
 //  * reads the fragments of the next 32 values of K before issuing the MFMAs of the current
 //    ones, with one barrier per stage placed in the middle of a stage, where the data of the
 //    next stage is known to have landed;
-//  * orders K inside a group of 32 so that a lane's 16 consecutive int8 feed two MFMAs: lanes
+//  * orders K inside a group of 32 so that a lane's 16 consecutive weights feed two MFMAs: lanes
 //    0-31 supply k = 0..7 then 8..15, lanes 32-63 supply 16..23 then 24..31, for W and x alike.
 // W is the MFMA "A" operand and x the "B" operand, so a lane ends up with four consecutive
 // output columns of one output row and stores them as 8 bytes.
