@@ -336,3 +336,35 @@ def test_batched_gemv_mode_stays_bit_exact(queue):
     q, s = mil.quantize_int8(W)
     got = _gemm(queue, M, N, K, X, q, s, "i8", tile=1)
     assert np.array_equal(got, O.gemm_i8(X, q, s.view(np.uint16)))
+
+
+def _random_shapes(seed, count):
+    rng = np.random.default_rng(seed)
+    shapes = [(2, 1, 64), (3, 7, 64), (16, 33, 128), (17, 255, 192), (31, 257, 64), (33, 1, 1024), (2, 300, 4864)]
+    while len(shapes) < count:
+        M = int(rng.choice([2, 3, 5, 15, 16, 17, 31, 32, 33, 63, 64, 65, 96, 127, 160, 161, 255, 300]))
+        N = int(rng.integers(1, 700))
+        K = 64 * int(rng.integers(1, 24))
+        shapes.append((M, N, K))
+    return shapes
+
+
+@pytest.mark.parametrize("kind", ["i8", "q4", "f16"])
+def test_gemm_random_shapes(queue, kind):
+    """Seeded shapes with ragged M and N (one row, one column, one more than a tile, ...), the
+    library's own choice of kernel and the wide kernel forced: within one fp16 step of the rows of GEMV."""
+    for i, (M, N, K) in enumerate(_random_shapes(77, 36)):
+        W, X = synth_w(3000 + i, N, K), synth_x(3100 + i, M, K)
+        for tile in (0, 3):
+            print(f"{kind} gemm M={M} N={N} K={K} mode {tile}", flush=True)
+            if kind == "i8":
+                q, s = mil.quantize_int8(W)
+                got, want = _gemm(queue, M, N, K, X, q, s, "i8", tile), O.gemm_i8(X, q, s.view(np.uint16))
+            elif kind == "q4":
+                p, s = mil.quantize_q4(W)
+                got, want = _gemm(queue, M, N, K, X, p, s, "q4", tile), O.gemm_q4(X, p, s.view(np.uint16))
+            else:
+                got, want = _gemm(queue, M, N, K, X, W, None, "f16", tile), O.gemm_f16(X, W)
+            assert_tolerance(got.view(np.float16), want.view(np.float16))
+            if not (kind == "q4" and tile == 0):
+                assert _ulp_apart(got, want).max() <= 1, (M, N, K, tile)
