@@ -215,13 +215,18 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const uint16_t* __restri
 namespace wide {
 
 constexpr int kBN = 256;                    // rows of W per block
-// LDS stages (K = 64 each) for 32 * tm rows of x: as many as 160 KB hold, at most 8.  A stage is
-// requested stages - 2 stage times before it is needed, which is what covers the load latency.
+// LDS stages (K = 64 each) for 32 * tm rows of x.  A stage is requested stages - 2 stage times
+// before it is needed, which is what covers the load latency.  Tall tiles (tm >= 3) take as many
+// stages as 160 KB hold.  Low tiles of quantised weights take half of the LDS (3 or 4 stages), so
+// that two blocks share a CU: they belong to shapes with many small tiles, where one block's
+// prologue and epilogue then overlap the other's main loop (lm_head at M = 16: 37 -> 29 us).
 constexpr int stages_for(int kind, int tm) {
-    return kind == WK_Q4 ? (tm >= 5 ? 5 : tm == 4 ? 6 : tm == 3 ? 7 : 8)
+    return kind == WK_Q4 ? (tm >= 5 ? 5 : tm == 4 ? 6 : tm == 3 ? 7 : 4)
          : kind == WK_F16 ? (tm >= 3 ? 3 : 4)
-                          : (tm >= 4 ? 4 : tm == 3 ? 5 : tm == 2 ? 6 : 8);
+                          : (tm >= 4 ? 4 : tm == 3 ? 5 : tm == 2 ? 3 : 4);
 }
+// blocks of such a tile that fit one CU
+constexpr int blocks_per_cu(int kind, int tm) { return kind != WK_F16 && tm <= 2 ? 2 : 1; }
 // bytes of W per stage: int8 rows of 64 bytes; fp16 rows of 128 bytes; Q4 rows of 32 bytes of
 // packed nibbles followed by the 256 rows' two block scales (fp16) each
 constexpr int w_stage_bytes(int kind) {
@@ -758,9 +763,17 @@ inline double estimate_us(int kind, int terms, int tm, int splits, int M, int N,
     const int stages = (K / 64 + splits - 1) / splits;
     const double stage_us = kind == WK_Q4 ? (terms == 2 ? 0.49 + 0.22 * tm : 0.56 + 0.10 * tm)
                           : kind == WK_F16 ? 0.35 + 0.10 * tm : 0.27 + 0.10 * tm;
-    const double block_us = 2.6 + 0.5 * tm + stages * stage_us;
-    const long full = blocks / cus, rem = blocks % cus;
-    double t = full * 1.56 * block_us + (rem ? (1.0 + 0.56 * rem / cus) * block_us : 0.0);
+    // two blocks on one CU take about 1.4 times as long each as one alone (the dispatcher puts a
+    // second block on a CU only when every CU has one)
+    const int per_cu = blocks > cus ? blocks_per_cu(kind, tm) : 1;
+    const double block_us = (2.6 + 0.5 * tm + stages * stage_us) * (per_cu == 2 ? 1.4 : 1.0);
+    const long slots = static_cast<long>(cus) * per_cu;
+    const long full = blocks / slots, rem = blocks % slots;
+    double t = full * 1.56 * block_us + (rem ? (1.0 + 0.56 * rem / slots) * block_us : 0.0);
+    // every row of tiles streams W again: not faster than that many bytes at about 6.4 TB/s
+    const double w_bytes = static_cast<double>((M + 32 * tm - 1) / (32 * tm)) * N * K *
+                           (kind == WK_F16 ? 2.0 : kind == WK_I8 ? 1.0 : 0.5625);
+    if (t < 2.5 + w_bytes / 6.4e6) t = 2.5 + w_bytes / 6.4e6;
     if (splits > 1) t += 2.5 + 2.0 * splits * M * static_cast<double>(N) * 4 / 4.0e6;   // ~4 TB/s there and back
     return t;
 }
