@@ -278,6 +278,16 @@ def main():
                     "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                     "frac_hbm": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
             mil.nnopt_unregister_weight(wb)
+        # a batch of 16 rows against the lm_head (batched decode): the weights stream once, as for one row
+        xb = mil.Buffer.from_host(mil.synth_normal_f16(78, 1.0, (16, H)))
+        ob = mil.Buffer(16 * VOCAB * 2)
+        arr = mil.make_calls([(16, VOCAB, H, xb, copies[i % 3][0], ob) for i in range(9)])
+        mil.linear_batch(queue, arr)
+        ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 5) / 9
+        nbytes = VOCAB * H + 2 * VOCAB + 2 * 16 * H + 2 * 16 * VOCAB
+        detail[f"c5_int8_gemm_M16_N{VOCAB}_K{H}"] = {
+            "us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+            "frac_hbm": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
         # the same contractions with fp16 weights
         for (N, K) in ((INTER, H), (H, INTER)):
             wb = mil.Buffer.from_host(mil.synth_normal_f16(77, 0.02, (N, K)))
