@@ -312,6 +312,24 @@ def test_q4_prefill_size_rows_sampled(queue):
     assert np.array_equal(got2[6], got[6])
 
 
+def test_fp16_prefill_size_rows_sampled(queue):
+    """Config 5 at M = 2048 with fp16 weights, both shapes: sampled rows equal the GEMV of that row of
+    x to one fp16 step; doubling a row of x doubles its output row exactly and leaves its neighbour alone."""
+    for (N, K) in ((4864, 896), (896, 4864)):
+        M = 2048
+        W, X = synth_w(2920 + N, N, K), synth_x(2921 + N, M, K)
+        got = _gemm(queue, M, N, K, X, W, None, "f16")
+        for r in [0, 1, 31, 32, 159, 160, 1000, 1023, 1024, 2046, 2047]:
+            want = O.gemv_f16(X[r], W)
+            assert _ulp_apart(got[r], want).max() <= 1, f"N={N} K={K} row {r}"
+        X2 = X.copy()
+        X2[5] = X[5] * np.float16(2.0)
+        got2 = _gemm(queue, M, N, K, X2, W, None, "f16")
+        normal = np.abs(got[5].view(np.float16)) >= np.float16(2.0 ** -13)      # (a subnormal fp16 output has fewer bits)
+        assert np.array_equal(got2[5].view(np.float16)[normal], (got[5].view(np.float16) * np.float16(2.0))[normal])
+        assert np.array_equal(got2[6], got[6])
+
+
 def test_prefill_size_rows_sampled(queue):
     """Config 5 at M = 2048: every sampled row of out equals the GEMV of that row of x."""
     M, N, K = 2048, 4864, 896
