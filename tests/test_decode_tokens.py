@@ -147,6 +147,29 @@ def test_smollm_widths_fp16_and_q4_weights_on_device(kind):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name,cfg,steps", [
+    ("long", dict(SMOL, max_pos=176, n_layers=2), 170),            # more keys than threads in the attention block
+    ("wide_heads", dict(hidden=1024, inter=1536, n_heads=8, n_kv_heads=2, head_dim=128, n_layers=2, vocab=2048,
+                        max_pos=80, rms_eps=1e-6, rope_theta=500000.0), 72),   # head_dim 128, K = 1024 / 1536
+    ("full_cache", dict(SMOL, max_pos=24, n_layers=1), 23),        # up to the last cache row
+])
+def test_device_step_other_geometries(name, cfg, steps):
+    """Long sequences, 128-wide heads and a cache filled to its last row: tokens and the last logits
+    of the device-only step equal the CPU harness's bit for bit."""
+    assert mil.lib().mi_init(0) == 1
+    queue = mil.Queue()
+    m = Model(cfg, seed=21)
+    want_logits = np.empty(cfg["vocab"], np.uint16)
+    want, _ = greedy(m, PROMPT[:1], steps, last_logits=want_logits)
+    gd = GpuDecoder(m, queue)
+    got = gd.greedy(PROMPT[:1], steps, graph=(name == "long"))
+    got_logits = gd.logits()
+    gd.close()
+    assert got == want
+    assert np.array_equal(got_logits, want_logits)
+
+
+@pytest.mark.gpu
 def test_one_layer_every_third_token_bit_identical():
     """One layer at SmolLM2 widths, one step at position 0 for 1366 different tokens: the residual
     stream behind the layer and the logits equal the CPU harness's bit for bit.  Each token is a
