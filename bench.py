@@ -378,9 +378,10 @@ def main():
         "metric": "quant GEMV achieved HBM GB/s (% of peak) + us/decode-step, Qwen2.5-0.5B shapes",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 weights, fp16 activations, fp32 accumulate", "data": "synthetic",
+        "dtype": "f32", "data": "synthetic",          # the sums; operands: int8 weights and fp16 scales, fp16 activations
         "config": {"workload": "Qwen2.5-0.5B decode-step matmul sweep, batch 1, per-row int8: 24 x "
                                "{q,k,v,o,gate,up,down} + lm_head = 169 GEMVs, 494873344 algorithmic bytes",
+                   "operands": "int8 weights with fp16 row scales, fp16 activations and outputs, fp32 accumulate",
                    "launch": launch_mode, "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
                    "us_per_decode_step": round(ms_step * 1e3, 1)},
         "roofline": roofline, "cpu_baseline": cpu, "detail": detail,
