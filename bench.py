@@ -214,6 +214,25 @@ def main():
         detail["c3_q4_gemv_151936x896"] = cold_gemv("q4", VOCAB, H, 4)
         detail["c3_int8_gemv_151936x896"] = {"us": roofline["us_per_launch"], "GBps": roofline["achieved"],
                                              "frac_hbm": roofline["frac"], "bytes": lm_bytes}
+        # the fused epilogues at the boundary (int8, warm): residual add, gate/up + SwiGLU, w3 + silu_mul
+        def fused_us(fn, n=32):
+            fn()
+            return round(time_region(mil, queue, lambda: [fn() for _ in range(n)], 5) / n * 1e3, 2)
+        wq = {}
+        for name, (N, K) in (("down", (H, INTER)), ("gate", (INTER, H)), ("up", (INTER, H))):
+            a_, b_ = mil.quantize_int8(mil.synth_normal_f16(300 + len(wq), 0.02, (N, K)))
+            wq[name] = (mil.Buffer.from_host(a_), mil.Buffer.from_host(b_))
+            assert mil.nnopt_register_int8_weight(wq[name][0], wq[name][1], N, K)
+        res_b, act_b = mil.Buffer(H * 2), mil.Buffer(INTER * 2)
+        detail["fused_int8_down_plus_residual_896x4864"] = {
+            "us_warm": fused_us(lambda: mil.pytorch_linear_add(queue, 1, H, INTER, x_i, wq["down"][0], res_b))}
+        detail["fused_int8_gate_up_silu_4864x896"] = {
+            "us_warm": fused_us(lambda: mil.fused_gate_up_silu_m1(queue, INTER, H, x_h, wq["gate"][0], wq["up"][0], act_b))}
+        detail["fused_int8_w3_silu_gate_4864x896"] = {
+            "us_warm": fused_us(lambda: mil.pytorch_linear_silu_gate_fused(queue, INTER, H, x_h, wq["up"][0], act_b))}
+        for wb_, _ in wq.values():
+            mil.nnopt_unregister_weight(wb_)
+
         # the greedy step's lm_head: GEMV + argmax, token left in device memory
         token = mil.Buffer(4)
 
