@@ -20,6 +20,7 @@
 // strided share of the logits to one candidate in scratch memory and a second, single-block
 // launch reduces those; without scratch memory one block does everything.
 #include "common.h"
+#include "argmax_rule.h"
 #include <hip/hip_fp16.h>
 
 namespace mi {
@@ -27,29 +28,7 @@ namespace {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kThreads = 256;
-constexpr float kNone = -3.402823466e+38f;
-
-struct Cand {
-    float v;
-    int i;
-};
-
-struct TieRule {
-    int chunk;      // elements per chunk: ceil(N / num_partials)
-    __device__ static unsigned rev6(int a) { return __brev(static_cast<unsigned>(a) & 63u) >> 26; }
-    __device__ bool before(int a, int b) const {          // a wins a tie against b
-        const int ca = a / chunk, cb = b / chunk;
-        if (ca != cb) return (ca & 63) != (cb & 63) ? rev6(ca) < rev6(cb) : ca < cb;
-        const int la = (a - ca * chunk) & 63, lb = (b - cb * chunk) & 63;
-        if (la != lb) return rev6(la) < rev6(lb);
-        return a < b;
-    }
-    __device__ Cand best(Cand a, Cand b) const {
-        if (b.v > a.v) return b;
-        if (a.v > b.v || !(b.v > kNone)) return a;         // the tie rule (two divisions) only for a real tie
-        return before(b.i, a.i) ? b : a;
-    }
-};
+constexpr float kNone = kArgmaxNone;
 
 __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
     return __half2float(__ushort_as_half(static_cast<unsigned short>(h)));
@@ -130,24 +109,57 @@ __global__ __launch_bounds__(kThreads) void argmax_f16_kernel(const uint16_t* __
     }
 }
 
-// The candidates of the kParts blocks to the token: one wavefront.
-__global__ __launch_bounds__(64) void argmax_finish_kernel(const float* __restrict__ part_v,
-                                                           const int* __restrict__ part_i, int parts, int N,
-                                                           int num_partials, int* __restrict__ out) {
+// Candidates (the kParts blocks' above, or the wavefronts' of a GEMV) to the token: one block of
+// 64 threads per 64 candidates, at most kFinishThreads.  A thread loads its first kAhead
+// candidates before it compares any: the launch is a chain of memory latencies otherwise.
+constexpr int kFinishThreads = 1024;
+__global__ __launch_bounds__(kFinishThreads) void argmax_finish_kernel(const float* __restrict__ part_v,
+                                                                 const int* __restrict__ part_i, int parts, int N,
+                                                                 int num_partials, int* __restrict__ out,
+                                                                 int* __restrict__ out2, int* __restrict__ counter) {
     const TieRule rule{(N + num_partials - 1) / num_partials};
     Cand c{kNone, 0};
-    for (int p = threadIdx.x; p < parts; p += 64) c = rule.best(c, Cand{part_v[p], part_i[p]});
+    constexpr int kAhead = 4;
+    Cand pre[kAhead];
     #pragma unroll
-    for (int s = 32; s > 0; s >>= 1) {
-        Cand o;
-        o.v = __shfl_down(c.v, s, 64);
-        o.i = __shfl_down(c.i, s, 64);
-        c = rule.best(c, o);
+    for (int u = 0; u < kAhead; ++u) {
+        const int p = threadIdx.x + u * blockDim.x;
+        pre[u] = p < parts ? Cand{part_v[p], part_i[p]} : Cand{kNone, 0};
     }
-    if (threadIdx.x == 0) out[0] = c.v > kNone ? c.i : 0;
+    #pragma unroll
+    for (int u = 0; u < kAhead; ++u) c = rule.best(c, pre[u]);
+    for (int p = threadIdx.x + kAhead * blockDim.x; p < parts; p += blockDim.x) c = rule.best(c, Cand{part_v[p], part_i[p]});
+    c = rule.best_of_wave(c);
+    __shared__ float sv[kFinishThreads / 64];
+    __shared__ int si[kFinishThreads / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    if (waves > 1) {
+        if (lane == 0) {
+            sv[wave] = c.v;
+            si[wave] = c.i;
+        }
+        __syncthreads();
+        if (wave != 0) return;
+        c = lane < waves ? Cand{sv[lane], si[lane]} : Cand{kNone, 0};
+        c = rule.best_of_wave(c);
+    }
+    if (threadIdx.x == 0) {
+        const int token = c.v > kNone ? c.i : 0;
+        out[0] = token;
+        if (out2) out2[0] = token;
+        if (counter) counter[0] = counter[0] + 1;
+    }
 }
 
 }  // namespace
+
+bool launch_argmax_finish(hipStream_t s, const float* cand_v, const int* cand_i, int count, int N, int num_partials,
+                          void* token_out, int* token_copy, int* counter) {
+    const int threads = count >= kFinishThreads ? kFinishThreads : (count + 63) / 64 * 64;
+    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(threads), 0, s, cand_v, cand_i, count, N, num_partials,
+                       static_cast<int*>(token_out), token_copy, counter);
+    return MI_HIP_OK(hipGetLastError());
+}
 
 bool launch_argmax_f16(hipStream_t s, const void* logits, int N, int num_partials, void* token_out,
                        void* scratch) {
@@ -162,7 +174,8 @@ bool launch_argmax_f16(hipStream_t s, const void* logits, int N, int num_partial
     auto* pi = reinterpret_cast<int*>(pv + kParts);
     hipLaunchKernelGGL(argmax_f16_kernel, dim3(kParts), dim3(kThreads), 0, s, x, N, num_partials, pv, pi, out);
     if (!MI_HIP_OK(hipGetLastError())) return false;
-    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(64), 0, s, pv, pi, kParts, N, num_partials, out);
+    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(64), 0, s, pv, pi, kParts, N, num_partials, out,
+                       static_cast<int*>(nullptr), static_cast<int*>(nullptr));
     return MI_HIP_OK(hipGetLastError());
 }
 

@@ -54,6 +54,12 @@ struct GemvCall {
     const void* norm_w = nullptr; // fp16 [K]: x is RMS-normalised with these weights first (M = 1, see gemv_takes_norm)
     float       norm_eps = 0.0f;
     int         add_mode = 0;         // EPI_ADD: an AddMode
+    // Greedy token: every wavefront of the launch also leaves the best (fp16 value, row) of the rows
+    // it computed, by the reference's argmax order for num_partials = am_np, in am_v / am_i
+    // [gemv_argmax_slots() entries]; one segment, M = 1, kernels of gemv_takes_norm only.
+    float*      am_v = nullptr;
+    int*        am_i = nullptr;
+    int         am_np = 0;
 };
 
 // gemv.hip
@@ -63,6 +69,9 @@ bool launch_gemv(hipStream_t s, const GemvCall& c);
 bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n);
 bool gemv_takes_norm(WeightKind kind, int K);    // GemvCall::norm_w is supported for this kind and K
 bool gemv_takes_swiglu(WeightKind kind, int K);  // EPI_SWIGLU is supported for this kind and K
+// Candidates a launch with GemvCall::am_v writes (one per wavefront of its grid), and their upper bound.
+int  gemv_argmax_slots(const GemvCall& c);
+constexpr int kGemvArgmaxMaxSlots = 8192;
 bool launch_gate_up_silu(hipStream_t s, WeightKind kind, int N, int K, const void* x,
                          const void* Wg, const void* sg, const void* Wu, const void* su, void* out);
 bool launch_dequant_int8(hipStream_t s, const void* q, const void* scale, int N, int K, void* w16);
@@ -74,12 +83,22 @@ bool launch_unpack_q4(hipStream_t s, const void* p, int N, int K, void* w8);
 // add behind (EPI_ADD: y[i] = fp16(fp16(W[i] x) + y[i])) or the SwiGLU of a gate / up pair (EPI_SWIGLU).
 bool fused_gemv(hipStream_t s, int n, const int* N, int K, const void* x, const void* const* W, void* const* y,
                 const void* norm_w, float norm_eps, Epilogue epi);
+// Logits of one x (RMS-normalised first when norm_w is not null) and their greedy token, the argmax
+// fused into the GEMV.  *taken = false, nothing launched: this weight kind, K or stream cannot, and the
+// caller runs the GEMV and launch_argmax_f16 itself.
+bool linear_argmax(hipStream_t s, int N, int K, const void* x, const void* W, void* logits, const void* norm_w,
+                   float norm_eps, int num_partials, void* token_out, int* token_copy, int* counter, bool* taken);
 bool fused_gemv_kind(const void* W, int N, int K, WeightKind* kind);   // kind W is registered as (fp16 if not)
 
 // argmax.hip: index of the greatest of N fp16 values, ties as the reference's two argmax kernels break them.
 // scratch: kArgmaxScratchBytes of device memory that belongs to stream s, or null (then one block does all the work).
 constexpr size_t kArgmaxScratchBytes = 512;
 bool launch_argmax_f16(hipStream_t s, const void* logits, int N, int num_partials, void* token_out, void* scratch);
+// The second step alone, over `count` candidates (value, index) left by another kernel (a GEMV with GemvCall::am_v).
+// token_copy, counter: null, or a second int the token is written to and an int that is incremented
+// (a decode step's "current token" and position, which saves the step a launch).
+bool launch_argmax_finish(hipStream_t s, const float* cand_v, const int* cand_i, int count, int N, int num_partials,
+                          void* token_out, int* token_copy, int* counter);
 
 // gemm.hip: out[M,N] = x[M,K] W^T on MFMA with the dequant fused into the tile load.
 // Shapes and pointers the GEMM kernels take (M >= 2, K a multiple of 64, 16-byte aligned x and W).

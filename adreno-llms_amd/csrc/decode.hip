@@ -490,13 +490,20 @@ int mi_decoder_step(void* dec, void* stream) {
         }
         if (!linear_into_h(c.inter, d->gate, d->wdown[l])) return 0;
     }
+    // (the fused argmax's second launch also does what advance_kernel does)
+    void* next = reinterpret_cast<char*>(d->st) + offsetof(State, next);
+    bool fused = false;
+    if (!linear_argmax(s, c.vocab, Hd, d->h, d->lm_head, d->logits, d->final_norm, c.rms_eps, 32, next, &d->st->token,
+                       &d->st->pos, &fused))
+        return 0;
+    if (fused) return 1;
     {
         const int N1[1] = {c.vocab};
         const void* const W1[1] = {d->lm_head};
         void* const y1[1] = {d->logits};
         if (!norm_linear(d->final_norm, 1, N1, W1, y1, false)) return 0;
+        if (!mi_argmax_f16(stream, d->logits, c.vocab, 32, next)) return 0;
     }
-    if (!mi_argmax_f16(stream, d->logits, c.vocab, 32, reinterpret_cast<char*>(d->st) + offsetof(State, next))) return 0;
     hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->st);
     return launched() ? 1 : 0;
 }

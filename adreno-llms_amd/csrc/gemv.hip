@@ -29,6 +29,7 @@
 #include "common.h"
 #include <hip/hip_fp16.h>
 #include "device_math.h"
+#include "argmax_rule.h"
 
 namespace mi {
 namespace {
@@ -59,6 +60,11 @@ struct SegList {
     const uint16_t* norm_w;   // not null: x is RMS-normalised with these weights before use
     float norm_eps;
     int add_mode;             // EPI_ADD: an AddMode
+    // not null: every wavefront of gemv_fixed_k leaves the best (fp16 value, row) of its rows here,
+    // slot = wavefront number in the grid, by the argmax order for chunks of am_chunk rows
+    float* am_v;
+    int* am_i;
+    int am_chunk;
 };
 
 // EPI_ADD, what happens to the value y already holds (res):
@@ -219,7 +225,7 @@ __device__ __forceinline__ Seg find_segment(const SegList& L, int rb) {
 // multiplies the current one.  Without PIPE a wavefront is expected to own one batch.
 // RB row batches are fetched together, so that narrow rows (Q4, small K) still keep enough
 // bytes in flight per wavefront.
-template <int KIND, int KT, int VL, int EPI, bool PIPE, int RB>
+template <int KIND, int KT, int VL, int EPI, bool PIPE, int RB, bool AM = false>
 __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restrict__ x, const SegList L) {
     using T = WT<KIND>;
     constexpr int LPR = kWave / VL, RPW = VL;
@@ -248,6 +254,7 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
         uint16_t res;
         uint16_t* ybase;    // &y[m][first row of the batch], uniform
         int yoff;           // row inside the batch, -1 when the lane's row is past N
+        int row0;           // first row of the batch inside its segment, uniform
     };
     const uint32_t lane_w = r * ROWB + koff / T::EPV * T::BPV;     // byte offset of the lane's weights
     const uint32_t lane_w0 = koff / T::EPV * T::BPV;               // same column, first row of the batch
@@ -260,6 +267,7 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
         const uint32_t wo = valid ? lane_w : lane_w0;
         b.ybase = sg.y + static_cast<size_t>(m) * sg.N + row0;
         b.yoff = valid ? r : -1;
+        b.row0 = row0;
         if constexpr (KIND == WK_I8) b.s[0] = (sg.sc + row0)[rr];
         if constexpr (EPI == EPI_ADD) b.res = b.ybase[rr];
         #pragma unroll
@@ -276,7 +284,15 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     // flight before anything waits.
     const int nw = gridDim.x * kWavesPerBlock;
     int rb = blockIdx.x * kWavesPerBlock + wave;
-    if (rb >= L.nbatch) return;
+    const int wid = rb;
+    const TieRule rule{L.am_chunk};
+    Cand top{kArgmaxNone, 0};                                 // AM: best row so far (lanes with g == 0)
+    if (rb >= L.nbatch) {
+        if constexpr (AM) {
+            if (lane == 0) { L.am_v[wid] = kArgmaxNone; L.am_i[wid] = 0; }
+        }
+        return;
+    }
     constexpr int GB = PIPE ? RB : 1;
     struct Group { Batch b[GB]; };
     const int first = rb;
@@ -393,7 +409,12 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
             } else {
                 out = EPI == EPI_ADD ? add_residual(sum, 1.0f, h_f(b.res), false, L.add_mode) : sum;
             }
-            b.ybase[b.yoff] = f_h(out);
+            const uint16_t bits = f_h(out);
+            b.ybase[b.yoff] = bits;
+            if constexpr (AM) {
+                const float v = h_f(bits);
+                if (v > kArgmaxNone) top = rule.best(top, Cand{v, b.row0 + b.yoff});
+            }
         }
     };
 
@@ -420,6 +441,10 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
             rb += step;
             if (rb >= L.nbatch) break;
         }
+    }
+    if constexpr (AM) {
+        const Cand w = rule.best_of_wave(top);
+        if (lane == 0) { L.am_v[wid] = w.v; L.am_i[wid] = w.i; }
     }
 }
 
@@ -772,6 +797,14 @@ Plan make_plan(const GemvCall* calls, int n, int vl) {
     p.L.norm_w = static_cast<const uint16_t*>(calls[0].norm_w);
     p.L.norm_eps = calls[0].norm_eps;
     p.L.add_mode = calls[0].add_mode;
+    p.L.am_v = nullptr;
+    p.L.am_i = nullptr;
+    p.L.am_chunk = 1;
+    if (calls[0].am_v && calls[0].am_np > 0) {
+        p.L.am_v = calls[0].am_v;
+        p.L.am_i = calls[0].am_i;
+        p.L.am_chunk = (calls[0].N + calls[0].am_np - 1) / calls[0].am_np;
+    }
     const int cap = resident_waves();
     int waves = first;
     p.pipe = false;
@@ -805,6 +838,29 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
             hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, false, 1>), p.grid, dim3(kBlock), 0, s, x, p.L); \
         }                                                                                                \
         break;
+    if constexpr (EPI == EPI_STORE && KIND != WK_Q4) {
+        if (p.L.am_v) {
+#define MI_FIXED_AM(KT, PIPE_OK)                                                                         \
+    case KT:                                                                                             \
+        if (PIPE_OK && p.pipe) {                                                                         \
+            constexpr int kRB = group_size(KIND, KT, VL);                                                \
+            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, PIPE_OK, kRB, true>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+        } else {                                                                                         \
+            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, false, 1, true>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+        }                                                                                                \
+        break;
+            switch (K) {
+                MI_FIXED_AM(576, true)
+                MI_FIXED_AM(896, true)
+                MI_FIXED_AM(1024, true)
+                MI_FIXED_AM(1536, true)
+                MI_FIXED_AM(4864, false)
+                default: MI_ERROR_FMT("gemv: no fused argmax for K=%d", K); return false;
+            }
+#undef MI_FIXED_AM
+            return MI_HIP_OK(hipGetLastError());
+        }
+    }
     switch (K) {
         MI_FIXED(576, true)
         MI_FIXED(896, true)
@@ -903,6 +959,11 @@ bool check_call(const GemvCall& c) {
 
 }  // namespace
 
+int gemv_argmax_slots(const GemvCall& c) {
+    const Plan p = make_plan(&c, 1, pick_vl(c.kind, c.M, c.N, c.K));
+    return static_cast<int>(p.grid.x) * kWavesPerBlock;
+}
+
 bool gemv_takes_swiglu(WeightKind kind, int K) {
     return (kind == WK_I8 || kind == WK_F16) && (K == 576 || K == 896 || K == 1024 || K == 1536);
 }
@@ -929,6 +990,11 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
         rows += calls[i].N;
     }
     const GemvCall& c = calls[0];
+    if (c.am_v && !(n == 1 && c.M == 1 && c.epi == EPI_STORE && c.am_i && c.am_np > 0 && gemv_takes_norm(c.kind, c.K))) {
+        MI_ERROR_FMT("gemv: the fused argmax takes one segment, M = 1, int8 or fp16 weights and a K kept in registers "
+                     "(kind=%d K=%d)", static_cast<int>(c.kind), c.K);
+        return false;
+    }
     if (c.norm_w && !(gemv_takes_norm(c.kind, c.K) && aligned(c.norm_w, 16))) {
         MI_ERROR_FMT("gemv: no fused RMSNorm for kind=%d K=%d (or misaligned norm weights)", static_cast<int>(c.kind), c.K);
         return false;

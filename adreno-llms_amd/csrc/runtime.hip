@@ -105,6 +105,27 @@ bool fused_gemv(hipStream_t s, int n, const int* N, int K, const void* x, const 
     return launch_gemv_group(s, group, n);
 }
 
+bool linear_argmax(hipStream_t s, int N, int K, const void* x, const void* W, void* logits, const void* norm_w,
+                   float norm_eps, int num_partials, void* token_out, int* token_copy, int* counter, bool* taken) {
+    *taken = false;
+    Entry e;
+    if (!resolve("linear_argmax", W, N, K, &e)) return false;
+    void* ws = workspace_of(s);
+    if (!ws || !gemv_takes_norm(e.kind, K)) return true;
+    GemvCall c;
+    c.x = x; c.W = W; c.scale = e.scale; c.y = logits;
+    c.M = 1; c.N = N; c.K = K; c.kind = e.kind; c.epi = EPI_STORE;
+    c.norm_w = norm_w; c.norm_eps = norm_eps;
+    static_assert(kGemvArgmaxMaxSlots * 8 <= kWorkspaceBytes, "candidates fit the workspace");
+    c.am_v = static_cast<float*>(ws);
+    c.am_i = reinterpret_cast<int*>(c.am_v + kGemvArgmaxMaxSlots);
+    c.am_np = num_partials;
+    const int slots = gemv_argmax_slots(c);
+    if (slots > kGemvArgmaxMaxSlots) return true;
+    *taken = true;
+    return launch_gemv(s, c) && launch_argmax_finish(s, c.am_v, c.am_i, slots, N, num_partials, token_out, token_copy, counter);
+}
+
 int gemv_mode() { return g_gemv_mode; }
 int gemm_mode() { return g_gemm_mode; }
 
@@ -293,6 +314,18 @@ int mi_argmax_f16(void* stream, const void* logits, int N, int num_partials, voi
 
 int mi_linear_argmax(void* stream, int N, int K, const void* x, const void* W, void* logits, int num_partials,
                      void* token_out) {
+    if (!ensure_init()) return 0;
+    if (N <= 0 || K <= 0 || !x || !W || !logits || !token_out || num_partials <= 0 ||
+        reinterpret_cast<uintptr_t>(token_out) % 4) {
+        MI_ERROR_FMT("mi_linear_argmax: bad argument (N=%d K=%d num_partials=%d token_out=%p)", N, K, num_partials,
+                     token_out);
+        return 0;
+    }
+    // One launch computes the logits and each wavefront's best row, a second reduces those; for
+    // the kernels that cannot (Q4, other K, a stream without workspace) the argmax reads the logits back.
+    bool taken = false;
+    if (!linear_argmax(as_stream(stream), N, K, x, W, logits, nullptr, 0.0f, num_partials, token_out, nullptr, nullptr, &taken)) return 0;
+    if (taken) return 1;
     if (!mi_linear(stream, 1, N, K, x, W, logits)) return 0;
     return mi_argmax_f16(stream, logits, N, num_partials, token_out);
 }

@@ -272,7 +272,7 @@ def main():
         pos_after, _ = dec.read(queue)
         detail["c4_whole_decode_step_on_device"] = {
             "us_per_token": round(ms_tok * 1e3, 1), "tokens_per_s": round(1e3 / ms_tok, 1),
-            "launches_per_step": 24 * 5 + 5, "positions": f"8..{pos_after - 1}", "launch": "hip_graph"}
+            "launches_per_step": 24 * 5 + 3, "positions": f"8..{pos_after - 1}", "launch": "hip_graph"}
         dec.close()
 
     # ---- config 5: prefill GEMM with fused int8 dequant on the matrix cores ---------------

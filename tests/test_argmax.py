@@ -139,6 +139,58 @@ def test_lm_head_then_argmax_on_device():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kind,N,K", [("int8", 151936, 896), ("fp16", 151936, 896), ("int8", 49152, 576),
+                                      ("fp16", 30001, 1536), ("int8", 5000, 4864), ("int8", 300, 1024),
+                                      ("q4", 20000, 896), ("int8", 7000, 640)])
+def test_argmax_inside_the_lm_head_launch(kind, N, K):
+    """Where the GEMV keeps x in registers (int8 and fp16, the K of the model families) its wavefronts
+    leave their best rows and a small launch picks the token from those; other kinds and K read the
+    logits back.  Either way: logits as mi_linear's, token as the oracle's from those logits, with
+    thousands of equal maxima (W has 40 distinct rows) and for several chunkings."""
+    from helpers import synth_w, synth_x
+    assert mil.lib().mi_init(0) == 1
+    q = mil.Queue()
+    rng = np.random.default_rng(N + K)
+    rows = synth_w(71, 40, K)
+    W = rows[rng.integers(0, 40, N)]
+    x = synth_x(72, 1, K).reshape(K)
+    xb = mil.Buffer.from_host(x)
+    if kind == "int8":
+        qw, s = mil.quantize_int8(W)
+        wb, sb = mil.Buffer.from_host(qw), mil.Buffer.from_host(s)
+        assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+    elif kind == "q4":
+        qw, s = mil.quantize_q4(W)
+        wb, sb = mil.Buffer.from_host(qw), mil.Buffer.from_host(s)
+        assert mil.nnopt_register_q4_weight(wb, sb, N, K)
+    else:
+        wb = mil.Buffer.from_host(W)
+    plain, logits = mil.Buffer(N * 2), mil.Buffer(N * 2)
+    tok = mil.Buffer.from_host(np.array([-1], np.int32))
+    try:
+        assert mil.pytorch_linear(q, 1, N, K, xb, wb, plain)
+        q.finish()
+        want_logits = plain.read(np.uint16, (N,))
+        v = want_logits.view(np.float16).astype(np.float32)
+        assert (v == v.max()).sum() >= max(2, min(20, N // 300))
+        for num_partials in (32, 1, 100, 257):
+            tok.write(np.array([-1], np.int32))
+            assert mil.pytorch_linear_argmax(q, N, K, xb, wb, logits, tok, num_partials)
+            q.finish()
+            assert np.array_equal(logits.read(np.uint16, (N,)), want_logits)
+            assert int(tok.read(np.int32, (1,))[0]) == O.argmax_f16(want_logits, num_partials), num_partials
+        # logits that are no candidates (x = -inf gives NaN and -inf only): token 0
+        xb2 = mil.Buffer.from_host(np.full(K, -np.inf, np.float16))
+        assert mil.pytorch_linear_argmax(q, N, K, xb2, wb, logits, tok)
+        q.finish()
+        got = logits.read(np.uint16, (N,))
+        assert int(tok.read(np.int32, (1,))[0]) == O.argmax_f16(got)
+    finally:
+        if kind != "fp16":
+            mil.nnopt_unregister_weight(wb)
+
+
+@pytest.mark.gpu
 def test_stream_without_workspace_takes_the_one_launch_paths():
     """A hipStream_t that mi_stream_create did not make has no workspace: the argmax runs as one
     block and an int8 GEMM that would cut K into slices runs unsliced.  Same results."""
