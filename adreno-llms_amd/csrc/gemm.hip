@@ -726,7 +726,14 @@ __global__ __launch_bounds__(256) void reduce_partials(const float* __restrict__
 
 template <int TM, int KIND, int TERMS>
 bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out,
-            float* partial, int splits) {
+            float* partial, size_t partial_bytes, int splits) {
+    // the kernel writes splits x M x N fp32 partial sums and gives every slice at least two K-stages
+    if (splits < 1 || (splits > 1 && (!partial || K / 64 < 2 * splits ||
+                                      static_cast<double>(splits) * M * N * 4 > static_cast<double>(partial_bytes)))) {
+        MI_ERROR_FMT("gemm: %d slices of K do not fit (M=%d N=%d K=%d, %zu bytes of workspace)", splits, M, N, K,
+                     partial_bytes);
+        return false;
+    }
     constexpr size_t lds_bytes = static_cast<size_t>(stages_for(KIND, TM)) * (32 * TM * 128 + w_stage_bytes(KIND));
     auto* kern = gemm_wide<TM, KIND, TERMS>;
     static bool raised = false;
@@ -770,9 +777,12 @@ inline double estimate_us(int kind, int terms, int tm, int splits, int M, int N,
     const long slots = static_cast<long>(cus) * per_cu;
     const long full = blocks / slots, rem = blocks % slots;
     double t = full * 1.56 * block_us + (rem ? (1.0 + 0.56 * rem / slots) * block_us : 0.0);
-    // every row of tiles streams W again: not faster than that many bytes at about 6.4 TB/s
-    const double w_bytes = static_cast<double>((M + 32 * tm - 1) / (32 * tm)) * N * K *
-                           (kind == WK_F16 ? 2.0 : kind == WK_I8 ? 1.0 : 0.5625);
+    // every row of tiles streams W again: not faster than that many bytes at about 6.4 TB/s, or,
+    // for a W that stays in the memory-side cache (32 MB taken as the limit), 2.2 times that for
+    // the reads after the first
+    const double w_once = static_cast<double>(N) * K * (kind == WK_F16 ? 2.0 : kind == WK_I8 ? 1.0 : 0.5625);
+    const int tiles_m = (M + 32 * tm - 1) / (32 * tm);
+    const double w_bytes = w_once <= 32.0e6 ? w_once * (1.0 + (tiles_m - 1) / 2.2) : w_once * tiles_m;
     if (t < 2.5 + w_bytes / 6.4e6) t = 2.5 + w_bytes / 6.4e6;
     if (splits > 1) t += 2.5 + 2.0 * splits * M * static_cast<double>(N) * 4 / 4.0e6;   // ~4 TB/s there and back
     return t;
@@ -797,13 +807,13 @@ inline void pick_shape(int kind, int terms, int M, int N, int K, int cus, size_t
 
 template <int KIND, int TERMS>
 bool launch_any(int tm, hipStream_t s, int M, int N, int K, const void* x, const void* W,
-                const void* scale, void* out, float* partial, int splits) {
+                const void* scale, void* out, float* partial, size_t partial_bytes, int splits) {
     switch (tm) {
-        case 1: return launch<1, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, splits);
-        case 2: return launch<2, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, splits);
-        case 3: return launch<3, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, splits);
-        case 4: return launch<4, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, splits);
-        default: return launch<5, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, splits);
+        case 1: return launch<1, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, partial_bytes, splits);
+        case 2: return launch<2, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, partial_bytes, splits);
+        case 3: return launch<3, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, partial_bytes, splits);
+        case 4: return launch<4, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, partial_bytes, splits);
+        default: return launch<5, KIND, TERMS>(s, M, N, K, x, W, scale, out, partial, partial_bytes, splits);
     }
 }
 
@@ -910,8 +920,8 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
         wide::pick_shape(WK_Q4, terms, M, N, K, cus, may_slice ? workspace_bytes : 0, &tm, &splits, nullptr);
         if (mode >= 11 && mode <= 15) tm = mode - 10;
         if (terms == 1)
-            return wide::launch_any<WK_Q4, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), splits);
-        return wide::launch_any<WK_Q4, 2>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), splits);
+            return wide::launch_any<WK_Q4, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), workspace ? workspace_bytes : 0, splits);
+        return wide::launch_any<WK_Q4, 2>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), workspace ? workspace_bytes : 0, splits);
     }
     if (wide_fits && (mode == 0 || mode == 3 || (mode >= 11 && mode <= 15))) {
         double wide_us = 0.0;
@@ -922,8 +932,8 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
         if (mode >= 11) tm = mode - 10;
         if (mode != 0 || wide_us < tiled_us) {
             if (kind == WK_F16)
-                return wide::launch_any<WK_F16, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), splits);
-            return wide::launch_any<WK_I8, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), splits);
+                return wide::launch_any<WK_F16, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), workspace ? workspace_bytes : 0, splits);
+            return wide::launch_any<WK_I8, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), workspace ? workspace_bytes : 0, splits);
         }
     } else if (mode == 3 || mode >= 11) {
         MI_ERROR_FMT("gemm: mode %d asks for the wide kernel, whose 32-bit offsets do not reach M=%d N=%d K=%d",
