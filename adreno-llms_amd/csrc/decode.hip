@@ -31,11 +31,20 @@ struct State {
 
 __device__ __forceinline__ float rcp_rn(float x) { return __fdiv_rn(1.0f, x); }
 
-// h[c] = embed[token][c]   (QW/kernels/embedding.cl)
+// h[c] = embed[token][c]   (QW/kernels/embedding.cl).  The first launch of a step also copies the
+// rotary table's row of the current position to rope_now (cosines, then sines: 2 D values), so
+// that the attention launches of the step find it without waiting for the position first.
 __global__ void embed_kernel(const uint16_t* __restrict__ embed, const State* __restrict__ st,
-                             uint16_t* __restrict__ h, int hidden, int vocab) {
+                             uint16_t* __restrict__ h, int hidden, int vocab, const uint16_t* __restrict__ cosT,
+                             const uint16_t* __restrict__ sinT, uint16_t* __restrict__ rope_now, int D, int max_pos) {
     int t = st->token;
     t = t < 0 ? 0 : (t >= vocab ? vocab - 1 : t);
+    int pos = st->pos;
+    pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+    for (int c = threadIdx.x; c < D; c += blockDim.x) {
+        rope_now[c] = cosT[static_cast<size_t>(pos) * D + c];
+        rope_now[D + c] = sinT[static_cast<size_t>(pos) * D + c];
+    }
     for (int c = threadIdx.x; c < hidden; c += blockDim.x) h[c] = embed[static_cast<size_t>(t) * hidden + c];
 }
 
@@ -245,6 +254,191 @@ __global__ __launch_bounds__(256) void rope_attention_kernel(const uint16_t* __r
     }
 }
 
+// The same launch for head widths known at compile time (64 and 128), laid out for latency: a
+// decode step at a short context is a chain of memory round trips, so everything that does not
+// depend on an earlier result is requested at once.  256 threads; the first kTileRows rows of the
+// group's key and value cache are requested in 16-byte pieces before anything else (rows past
+// the current position too: the caches hold max_pos rows, and what is not older than the current
+// position is never used), then the projections, biases and the rotary row (which the step's first
+// launch has set aside, so that its address does not wait for the position); keys and values wait
+// in LDS tiles (rows padded by 16 bytes against bank conflicts) while q, k and v of the current
+// position are prepared.  Scores: one thread per key from the tile; values: one thread per
+// output element, keys in index order from the tile.  Longer contexts take further tiles the
+// same way, one round trip per 128 rows.  The arithmetic and its order are those of
+// rope_attention_kernel.
+// Dynamic LDS: 6 D bytes, 6 bytes per position, rounded up to 16, then two tiles of
+// kTileRows x (2 D + 16) bytes.
+constexpr int kTileRows = 128;
+constexpr int kMaxPositions = 8192;                      // longest context a decoder is created for
+
+template <int D>
+__global__ __launch_bounds__(256) void rope_attention_tiled(const uint16_t* __restrict__ q_raw, const uint16_t* __restrict__ k_raw,
+                                      const uint16_t* __restrict__ v_raw, const uint16_t* __restrict__ bq,
+                                      const uint16_t* __restrict__ bk, const uint16_t* __restrict__ bv,
+                                      const uint16_t* __restrict__ rope_now,
+                                      uint16_t* __restrict__ kc, uint16_t* __restrict__ vc,
+                                      uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_out,
+                                      uint16_t* __restrict__ v_out, uint16_t* __restrict__ out,
+                                      const State* __restrict__ st, int n_heads, int n_kv_heads, int max_pos,
+                                      float scale) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    constexpr int kRowH = D + 8;                           // tile row stride in halves
+    constexpr int kPieces = D / 8;                         // 16-byte pieces per row
+    constexpr int kPasses = kTileRows * kPieces / 256;     // pieces per thread and tile
+    static_assert(kTileRows * kPieces % 256 == 0, "whole passes");
+    extern __shared__ __attribute__((aligned(16))) uint16_t qv[];
+    uint16_t* kcur = qv + D;
+    uint16_t* vcur = kcur + D;
+    float* ex = reinterpret_cast<float*>(vcur + D);                        // [max_pos] exponentials
+    uint16_t* sc = reinterpret_cast<uint16_t*>(ex + max_pos);              // [max_pos] scores
+    uint16_t* ktile = qv + ((3 * D + 3 * max_pos + 7) & ~7);               // 16-byte aligned
+    uint16_t* vtile = ktile + kTileRows * kRowH;
+    const int nrep = n_heads / n_kv_heads;
+    const int qh = blockIdx.x, kvd = n_kv_heads * D, kvh = qh / nrep, hd2 = D / 2;
+    const bool writer = qh % nrep == 0;
+    const int tid = threadIdx.x;
+
+    // piece p of this thread in a tile: row (tid + 256 p) / kPieces, 16-byte piece (tid + 256 p) % kPieces
+    auto request = [&](const uint16_t* cache, int row0, u32x4 (&r)[kPasses]) {
+        #pragma unroll
+        for (int p = 0; p < kPasses; ++p) {
+            const int idx = tid + 256 * p, row = idx / kPieces, piece = idx % kPieces;
+            const int tk = row0 + row < max_pos ? row0 + row : max_pos - 1;
+            r[p] = *reinterpret_cast<const u32x4*>(cache + static_cast<size_t>(tk) * kvd + kvh * D + 8 * piece);
+        }
+    };
+    auto keep = [&](uint16_t* tile, const u32x4 (&r)[kPasses]) {
+        #pragma unroll
+        for (int p = 0; p < kPasses; ++p) {
+            const int idx = tid + 256 * p, row = idx / kPieces, piece = idx % kPieces;
+            *reinterpret_cast<u32x4*>(tile + row * kRowH + 8 * piece) = r[p];
+        }
+    };
+    u32x4 kreg[kPasses], vreg[kPasses];
+    request(kc, 0, kreg);
+    request(vc, 0, vreg);
+
+    int pos = st->pos;
+    pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+    const int seq_k = pos + 1;
+    const uint16_t* cr = rope_now;                          // the rotary row of this position (embed_kernel)
+    const uint16_t* sr = rope_now + D;
+    if (tid < hd2) {
+        const int i = tid;
+        const float c = h_f(cr[i]), sn = h_f(sr[i]);
+        {
+            const uint16_t* buf = q_raw + qh * D;
+            const uint16_t* bias = bq + qh * D;
+            const float x1 = h_f(f_h(h_f(buf[i]) + h_f(bias[i])));
+            const float x2 = h_f(f_h(h_f(buf[i + hd2]) + h_f(bias[i + hd2])));
+            const uint16_t r1 = f_h(fmaf(x1, c, -(x2 * sn))), r2 = f_h(fmaf(x2, c, x1 * sn));
+            qv[i] = r1;
+            qv[i + hd2] = r2;
+            q_out[qh * D + i] = r1;
+            q_out[qh * D + i + hd2] = r2;
+        }
+    } else if (tid >= 64 && tid < 64 + hd2) {
+        const int i = tid - 64;
+        const float c = h_f(cr[i]), sn = h_f(sr[i]);
+        const uint16_t* buf = k_raw + kvh * D;
+        const uint16_t* bias = bk + kvh * D;
+        const float x1 = h_f(f_h(h_f(buf[i]) + h_f(bias[i])));
+        const float x2 = h_f(f_h(h_f(buf[i + hd2]) + h_f(bias[i + hd2])));
+        const uint16_t r1 = f_h(fmaf(x1, c, -(x2 * sn))), r2 = f_h(fmaf(x2, c, x1 * sn));
+        kcur[i] = r1;
+        kcur[i + hd2] = r2;
+        if (writer) {
+            uint16_t* dst = kc + static_cast<size_t>(pos) * kvd + kvh * D;
+            dst[i] = r1;
+            dst[i + hd2] = r2;
+            k_out[kvh * D + i] = r1;
+            k_out[kvh * D + i + hd2] = r2;
+        }
+    } else if (tid >= 128 && tid < 128 + D) {
+        const int e = tid - 128;
+        const uint16_t r = f_h(h_f(v_raw[kvh * D + e]) + h_f(bv[kvh * D + e]));
+        vcur[e] = r;
+        if (writer) {
+            vc[static_cast<size_t>(pos) * kvd + kvh * D + e] = r;
+            v_out[kvh * D + e] = r;
+        }
+    }
+    keep(ktile, kreg);
+    keep(vtile, vreg);
+    __syncthreads();
+
+    // scores: tile rows by threads 0 .. kTileRows - 1, the current position by thread kTileRows
+    auto score = [&](const uint16_t* krow) {
+        typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+        const u16x4* kv = reinterpret_cast<const u16x4*>(krow);
+        const u16x4* qq = reinterpret_cast<const u16x4*>(qv);
+        float acc = 0.0f;
+        #pragma unroll
+        for (int d4 = 0; d4 < D / 4; ++d4) {
+            const u16x4 a = qq[d4], b = kv[d4];
+            float t = h_f(a[0]) * h_f(b[0]);
+            t = fmaf(h_f(a[1]), h_f(b[1]), t);
+            t = fmaf(h_f(a[2]), h_f(b[2]), t);
+            t = fmaf(h_f(a[3]), h_f(b[3]), t);
+            acc = acc + t;
+        }
+        return f_h(acc * scale);
+    };
+    if (tid == kTileRows) sc[pos] = score(kcur);
+    for (int row0 = 0; row0 < pos; row0 += kTileRows) {
+        if (row0 > 0) {
+            request(kc, row0, kreg);
+            __syncthreads();                               // the previous tile's scores are done
+            keep(ktile, kreg);
+            __syncthreads();
+        }
+        if (tid < kTileRows && row0 + tid < pos) sc[row0 + tid] = score(ktile + tid * kRowH);
+    }
+    __syncthreads();
+    // softmax by the first wavefront alone: its LDS accesses are ordered, so the steps need no
+    // barrier between them (a short context is all barrier otherwise)
+    if (tid < 64) {
+        float m = -3.402823466e+38f;                       // maximum: any order gives the same value
+        for (int c = tid; c < seq_k; c += 64) m = fmaxf(m, h_f(sc[c]));
+        for (int s = 32; s > 0; s >>= 1) m = fmaxf(m, __shfl_xor(m, s, 64));
+        const float maxv = m;
+        for (int c = tid; c < seq_k; c += 64) {
+            const float e = exp_poly(h_f(sc[c]) - maxv);
+            ex[c] = e;
+            sc[c] = f_h(e);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");  // lane 0 reads what the other lanes wrote
+        __builtin_amdgcn_wave_barrier();
+        float inv = 0.0f;
+        if (tid == 0) {
+            float sum = 0.0f;
+            for (int c = 0; c < seq_k; ++c) sum = sum + ex[c];
+            inv = rcp_rn(sum + 1e-20f);
+        }
+        inv = __shfl(inv, 0, 64);
+        for (int c = tid; c < seq_k; c += 64) sc[c] = f_h(h_f(sc[c]) * inv);
+    }
+    __syncthreads();
+    // output element e by thread e: older keys in index order from the tiles, then the current one
+    float acc = 0.0f;
+    for (int row0 = 0; row0 < pos; row0 += kTileRows) {
+        if (row0 > 0) {
+            request(vc, row0, vreg);
+            __syncthreads();                               // the previous tile has been used up
+            keep(vtile, vreg);
+            __syncthreads();
+        }
+        if (tid < D) {
+            const int n = pos - row0 < kTileRows ? pos - row0 : kTileRows;
+            for (int r = 0; r < n; ++r) acc = fmaf(h_f(sc[row0 + r]), h_f(vtile[r * kRowH + tid]), acc);
+        }
+    }
+    if (tid < D) {
+        acc = fmaf(h_f(sc[pos]), h_f(vcur[tid]), acc);
+        out[qh * D + tid] = f_h(acc);
+    }
+}
+
 // gate[i] = fp16((g * sigmoid(g)) * up[i])   (QW/kernels/mlp.cl swiglu_inplace)
 __global__ void swiglu_kernel(uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, int n) {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
@@ -252,6 +446,12 @@ __global__ void swiglu_kernel(uint16_t* __restrict__ gate, const uint16_t* __res
         const float sig = rcp_rn(1.0f + exp_poly(-g));
         gate[i] = f_h((g * sig) * u);
     }
+}
+
+// Dynamic LDS of rope_attention_tiled<D>.
+inline size_t tiled_attention_lds(int D, int max_pos) {
+    const size_t head = (static_cast<size_t>(3 * D + 3 * max_pos + 7) & ~static_cast<size_t>(7)) * 2;
+    return head + 2 * static_cast<size_t>(kTileRows) * (D + 8) * 2;
 }
 
 __global__ void advance_kernel(State* st) {
@@ -269,6 +469,7 @@ struct Decoder {
     uint16_t *kc = nullptr, *vc = nullptr, *cosT = nullptr, *sinT = nullptr;
     uint16_t *h = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr;
     uint16_t *qr = nullptr, *kr = nullptr, *vr = nullptr;      // q, k, v after bias and rotary embedding
+    uint16_t* rope_now = nullptr;                              // cosines and sines of the current position (embed_kernel)
     uint16_t *gate = nullptr, *up = nullptr, *logits = nullptr;
     State* st = nullptr;
     std::vector<void*> owned;
@@ -296,7 +497,7 @@ void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* 
     if (!cfg || !w || mi_init(0) != 1) return nullptr;
     const mi_decoder_config& c = *cfg;
     if (c.hidden <= 0 || c.inter <= 0 || c.n_heads <= 0 || c.n_kv_heads <= 0 || c.head_dim <= 0 || c.n_layers <= 0 ||
-        c.vocab <= 0 || c.max_pos <= 0 || c.n_heads % c.n_kv_heads || c.head_dim % 4 || c.head_dim > 256 || c.max_pos > 8192) {
+        c.vocab <= 0 || c.max_pos <= 0 || c.n_heads % c.n_kv_heads || c.head_dim % 4 || c.head_dim > 256 || c.max_pos > kMaxPositions) {
         MI_ERROR_FMT("mi_decoder_create: bad configuration");
         return nullptr;
     }
@@ -322,6 +523,16 @@ void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* 
     }
 
     const int D = c.head_dim, kvd = c.n_kv_heads * D, qd = c.n_heads * D;
+    if (D == 64 || D == 128) {
+        // more than 64 KB of LDS per block has to be asked for once per kernel: the most any context length needs
+        const size_t most = tiled_attention_lds(D, kMaxPositions);
+        const void* kern = D == 64 ? reinterpret_cast<const void*>(rope_attention_tiled<64>)
+                                   : reinterpret_cast<const void*>(rope_attention_tiled<128>);
+        if (!MI_HIP_OK(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(most)))) {
+            delete d;
+            return nullptr;
+        }
+    }
     const size_t cache = static_cast<size_t>(L) * c.max_pos * kvd * 2;
     bool ok = dev_alloc(d, &d->kc, cache) && dev_alloc(d, &d->vc, cache) &&
               dev_alloc(d, &d->cosT, static_cast<size_t>(c.max_pos) * D * 2) &&
@@ -331,7 +542,7 @@ void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* 
               dev_alloc(d, &d->kr, kvd * 2) && dev_alloc(d, &d->vr, kvd * 2) && dev_alloc(d, &d->attn, qd * 2) &&
               dev_alloc(d, &d->gate, c.inter * 2) &&
               dev_alloc(d, &d->up, c.inter * 2) && dev_alloc(d, &d->logits, static_cast<size_t>(c.vocab) * 2) &&
-              dev_alloc(d, &d->st, sizeof(State));
+              dev_alloc(d, &d->st, sizeof(State)) && dev_alloc(d, &d->rope_now, 2 * D * 2);
     if (ok) {
         // rotary tables, QW/src/layers/attention.cpp:133-172: cos/sin(t * theta^(-2i/D)), both halves alike
         std::vector<uint16_t> ct(static_cast<size_t>(c.max_pos) * D), stb(ct.size());
@@ -464,7 +675,8 @@ int mi_decoder_step(void* dec, void* stream) {
         void* const y1[1] = {d->h};
         return fused_gemv(s, 1, N1, K, x, W1, y1, nullptr, 0.0f, EPI_ADD);
     };
-    hipLaunchKernelGGL(embed_kernel, dim3(1), dim3(256), 0, s, static_cast<const uint16_t*>(d->embed), d->st, d->h, Hd, c.vocab);
+    hipLaunchKernelGGL(embed_kernel, dim3(1), dim3(256), 0, s, static_cast<const uint16_t*>(d->embed), d->st, d->h, Hd, c.vocab,
+                       d->cosT, d->sinT, d->rope_now, D, c.max_pos);
     if (!launched()) return 0;
     for (int l = 0; l < c.n_layers; ++l) {
         {
@@ -475,11 +687,24 @@ int mi_decoder_step(void* dec, void* stream) {
         }
         uint16_t* kc = d->kc + static_cast<size_t>(l) * c.max_pos * kvd;
         uint16_t* vc = d->vc + static_cast<size_t>(l) * c.max_pos * kvd;
-        const int at = D > 64 ? D : 64;
-        hipLaunchKernelGGL(rope_attention_kernel, dim3(c.n_heads), dim3(at), static_cast<size_t>(c.max_pos) * 6 + D * 6, s,
-                           d->q, d->k, d->v, static_cast<const uint16_t*>(d->bq[l]), static_cast<const uint16_t*>(d->bk[l]),
-                           static_cast<const uint16_t*>(d->bv[l]), d->cosT, d->sinT, kc, vc, d->qr, d->kr, d->vr, d->attn,
-                           d->st, c.n_heads, c.n_kv_heads, D, c.max_pos, scale);
+        const auto *bq = static_cast<const uint16_t*>(d->bq[l]), *bk = static_cast<const uint16_t*>(d->bk[l]),
+                   *bv = static_cast<const uint16_t*>(d->bv[l]);
+        if (D == 64 || D == 128) {
+            const size_t lds = tiled_attention_lds(D, c.max_pos);
+            if (D == 64)
+                hipLaunchKernelGGL(rope_attention_tiled<64>, dim3(c.n_heads), dim3(256), lds, s, d->q, d->k, d->v, bq, bk, bv,
+                                   d->rope_now, kc, vc, d->qr, d->kr, d->vr, d->attn, d->st, c.n_heads, c.n_kv_heads,
+                                   c.max_pos, scale);
+            else
+                hipLaunchKernelGGL(rope_attention_tiled<128>, dim3(c.n_heads), dim3(256), lds, s, d->q, d->k, d->v, bq, bk, bv,
+                                   d->rope_now, kc, vc, d->qr, d->kr, d->vr, d->attn, d->st, c.n_heads, c.n_kv_heads,
+                                   c.max_pos, scale);
+        } else {
+            const int at = D > 64 ? D : 64;
+            hipLaunchKernelGGL(rope_attention_kernel, dim3(c.n_heads), dim3(at), static_cast<size_t>(c.max_pos) * 6 + D * 6, s,
+                               d->q, d->k, d->v, bq, bk, bv, d->cosT, d->sinT, kc, vc, d->qr, d->kr, d->vr, d->attn,
+                               d->st, c.n_heads, c.n_kv_heads, D, c.max_pos, scale);
+        }
         if (!launched()) return 0;
         if (!linear_into_h(qd, d->attn, d->wo[l])) return 0;
         {

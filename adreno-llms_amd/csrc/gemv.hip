@@ -280,8 +280,6 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
                 b.s[j] = (sg.sc + static_cast<size_t>(row0) * (KT / 32))[rr * (KT / 32) + (active ? j * 16 + (g * VL) / 4 : 0)];
         }
     };
-    // Order of issue: the first group of row batches, then the activations: both are in
-    // flight before anything waits.
     const int nw = gridDim.x * kWavesPerBlock;
     int rb = blockIdx.x * kWavesPerBlock + wave;
     const int wid = rb;
@@ -304,10 +302,9 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
         for (int u = 0; u < GB; ++u) fetch(gr.b[u], at + u * nw < L.nbatch ? at + u * nw : first);
     };
     const int step = nw * GB;
-    Group g0, g1;
-    fetch_group(g0, rb);
-    if constexpr (EPI == EPI_SWIGLU) fetch(g1.b[0], rb + L.s[1].first);
-
+    // x (and the norm weights) are requested first and the first weights right behind them,
+    // without a wait in between: loads return in order, so the norm of x can start while the
+    // weights are still on their way, and not the other way round.
     uint32_t xr[NIT][XD];
     #pragma unroll
     for (int j = 0; j < NIT; ++j) {
@@ -317,6 +314,17 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
             for (int i = 0; i < XD; ++i) xr[j][i] = 0u;
         }
     }
+    [[maybe_unused]] uint32_t nrm[NIT][XD];
+    if constexpr (T::EPV == 4) {
+        if (L.norm_w) {
+            #pragma unroll
+            for (int j = 0; j < NIT; ++j)
+                load_dwords<XD, false>(nrm[j], L.norm_w + (j * EIT + koff < KT ? j * EIT + koff : koff));
+        }
+    }
+    Group g0, g1;
+    fetch_group(g0, rb);
+    if constexpr (EPI == EPI_SWIGLU) fetch(g1.b[0], rb + L.s[1].first);
 
     // RMSNorm of x in place of a kernel of its own (QW/kernels/rmsnorm.cl: 64 lanes, each summing
     // the squares of elements 4 lane + 256 j, the same tree as the GEMV's, then
@@ -324,10 +332,6 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     // wavefront repeats the sum in the reference's order while its first weights are in flight.
     if constexpr (T::EPV == 4) {
         if (L.norm_w) {
-            uint32_t nw[NIT][XD];
-            #pragma unroll
-            for (int j = 0; j < NIT; ++j)
-                load_dwords<XD, false>(nw[j], L.norm_w + (j * EIT + koff < KT ? j * EIT + koff : koff));
             float part[VL];
             #pragma unroll
             for (int v = 0; v < VL; ++v) part[v] = 0.0f;
@@ -353,8 +357,8 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
             for (int j = 0; j < NIT; ++j) {
                 #pragma unroll
                 for (int i = 0; i < XD; ++i) {
-                    const uint32_t lo = f_h((lo_f(xr[j][i]) * inv) * lo_f(nw[j][i]));
-                    const uint32_t hi = f_h((hi_f(xr[j][i]) * inv) * hi_f(nw[j][i]));
+                    const uint32_t lo = f_h((lo_f(xr[j][i]) * inv) * lo_f(nrm[j][i]));
+                    const uint32_t hi = f_h((hi_f(xr[j][i]) * inv) * hi_f(nrm[j][i]));
                     xr[j][i] = lo | (hi << 16);
                 }
             }
@@ -999,9 +1003,10 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
         MI_ERROR_FMT("gemv: no fused RMSNorm for kind=%d K=%d (or misaligned norm weights)", static_cast<int>(c.kind), c.K);
         return false;
     }
-    // (SwiGLU: a wavefront takes a row batch of both matrices, so there are half as many
-    //  wavefronts as batches; the lane tile is picked for that count)
-    const int vl = pick_vl(c.kind, c.M, c.epi == EPI_SWIGLU ? rows / 4 : rows, c.K);
+    // (SwiGLU: a wavefront takes a row batch of both matrices, and the launch is short: the
+    //  narrow tiles win until there are two batch pairs per wavefront and more.  Measured in a
+    //  decode step at 2 x 4864 rows, K = 896: one row per wavefront 4 % faster per token than two)
+    const int vl = pick_vl(c.kind, c.M, c.epi == EPI_SWIGLU ? rows / 8 : rows, c.K);
     if (c.epi == EPI_SWIGLU) {
         if (n != 2 || calls[0].N != calls[1].N || c.M != 1 || !gemv_takes_swiglu(c.kind, c.K)) {
             MI_ERROR_FMT("gemv: the SwiGLU epilogue takes a gate and an up matrix of equal N, M = 1, int8 or fp16 "
