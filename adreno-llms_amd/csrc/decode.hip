@@ -400,8 +400,7 @@ __global__ __launch_bounds__(256) void rope_attention_tiled(const uint16_t* __re
     if (tid < 64) {
         float m = -3.402823466e+38f;                       // maximum: any order gives the same value
         for (int c = tid; c < seq_k; c += 64) m = fmaxf(m, h_f(sc[c]));
-        for (int s = 32; s > 0; s >>= 1) m = fmaxf(m, __shfl_xor(m, s, 64));
-        const float maxv = m;
+        const float maxv = wave_max(m);
         for (int c = tid; c < seq_k; c += 64) {
             const float e = exp_poly(h_f(sc[c]) - maxv);
             ex[c] = e;
@@ -415,7 +414,7 @@ __global__ __launch_bounds__(256) void rope_attention_tiled(const uint16_t* __re
             for (int c = 0; c < seq_k; ++c) sum = sum + ex[c];
             inv = rcp_rn(sum + 1e-20f);
         }
-        inv = __shfl(inv, 0, 64);
+        inv = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(inv)));
         for (int c = tid; c < seq_k; c += 64) sc[c] = f_h(h_f(sc[c]) * inv);
     }
     __syncthreads();

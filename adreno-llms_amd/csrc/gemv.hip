@@ -188,8 +188,8 @@ template <int VL> __device__ __forceinline__ float reduce_row(float (&acc)[VL]) 
     constexpr int LPR = kWave / VL;
     #pragma unroll
     for (int v = 0; v < VL; ++v) {
-        if constexpr (LPR >= 64) acc[v] = acc[v] + __shfl_down(acc[v], 32, 64);
-        if constexpr (LPR >= 32) acc[v] = acc[v] + __shfl_down(acc[v], 16, LPR);
+        if constexpr (LPR >= 64) acc[v] = acc[v] + lane_plus32(acc[v]);
+        if constexpr (LPR >= 32) acc[v] = acc[v] + lane_plus16(acc[v]);
     }
     #pragma unroll
     for (int v = 0; v < VL; ++v) acc[v] = add_from_above<8>(acc[v]);
