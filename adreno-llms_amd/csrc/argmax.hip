@@ -75,13 +75,7 @@ __global__ __launch_bounds__(kThreads) void argmax_f16_kernel(const uint16_t* __
     for (int i = lead + 8 * groups + tid; i < N; i += nthreads) offer(half_bits_to_float(x[i]), i);
 
     // wavefront, then block
-    #pragma unroll
-    for (int s = 32; s > 0; s >>= 1) {
-        Cand o;
-        o.v = __shfl_down(c.v, s, 64);
-        o.i = __shfl_down(c.i, s, 64);
-        c = rule.best(c, o);
-    }
+    c = rule.best_of_wave(c);
     __shared__ float sv[kThreads / 64];
     __shared__ int si[kThreads / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -92,13 +86,7 @@ __global__ __launch_bounds__(kThreads) void argmax_f16_kernel(const uint16_t* __
     __syncthreads();
     if (wave == 0) {
         Cand r = lane < kThreads / 64 ? Cand{sv[lane], si[lane]} : Cand{kNone, 0};
-        #pragma unroll
-        for (int s = kThreads / 128; s > 0; s >>= 1) {
-            Cand o;
-            o.v = __shfl_down(r.v, s, 64);
-            o.i = __shfl_down(r.i, s, 64);
-            r = rule.best(r, o);
-        }
+        r = rule.best_of_wave(r);
         if (lane != 0) return;
         if (part_v) {
             part_v[blockIdx.x] = r.v;

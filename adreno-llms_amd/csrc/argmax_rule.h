@@ -5,6 +5,7 @@
 // index.  A logit is a candidate only if it is greater than -FLT_MAX (NaN and -inf never are).
 #pragma once
 #include <hip/hip_runtime.h>
+#include "device_math.h"
 
 namespace mi {
 
@@ -30,15 +31,22 @@ struct TieRule {
         if (a.v > b.v || !(b.v > kArgmaxNone)) return a;   // the tie rule (two divisions) only for a real tie
         return before(b.i, a.i) ? b : a;
     }
-    // the best of a wavefront's 64 candidates, in lane 0
+    // the best of a wavefront's 64 candidates, in lane 0: lane g takes in lane g + 32, + 16
+    // (register moves), then + 8 .. + 1 inside its row of 16 (DPP row shifts); a lane without
+    // such a partner meets its own candidate, which changes nothing
+    template <int SH> __device__ static Cand from_above(Cand c) {
+        Cand o;
+        o.v = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(c.v), __float_as_int(c.v), 0x100 + SH, 0xf, 0xf, false));
+        o.i = __builtin_amdgcn_update_dpp(c.i, c.i, 0x100 + SH, 0xf, 0xf, false);
+        return o;
+    }
     __device__ Cand best_of_wave(Cand c) const {
-        #pragma unroll
-        for (int s = 32; s > 0; s >>= 1) {
-            Cand o;
-            o.v = __shfl_down(c.v, s, 64);
-            o.i = __shfl_down(c.i, s, 64);
-            c = best(c, o);
-        }
+        c = best(c, Cand{lane_plus32(c.v), __float_as_int(lane_plus32(__int_as_float(c.i)))});
+        c = best(c, Cand{lane_plus16(c.v), __float_as_int(lane_plus16(__int_as_float(c.i)))});
+        c = best(c, from_above<8>(c));
+        c = best(c, from_above<4>(c));
+        c = best(c, from_above<2>(c));
+        c = best(c, from_above<1>(c));
         return c;
     }
 };
