@@ -506,11 +506,21 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
             b.s[j] = sb[rr * (KT / 32) + (active ? j * 16 + g : 0)];
         }
     };
-    // The first weights are requested before the activations: the pairing of x below waits
-    // for x to arrive, and that wait should not delay the first fetch by a memory latency.
+    // The activations are requested first and the first weights right behind them, without a
+    // wait in between: loads return in order, so the pairing of x below can run while the
+    // weights are still on their way.
     const int nw = gridDim.x * kWavesPerBlock;
     int rb = blockIdx.x * kWavesPerBlock + wave;
     if (rb >= L.nbatch) return;
+    uint32_t raw[NIT][16];
+    #pragma unroll
+    for (int j = 0; j < NIT; ++j) {
+        if (j * EIT + koff < KT) load_dwords<16, false>(raw[j], x + j * EIT + koff);
+        else {
+            #pragma unroll
+            for (int i = 0; i < 16; ++i) raw[j][i] = 0u;
+        }
+    }
     struct Group { Batch b[PIPE ? RB : 1]; };
     constexpr int GB = PIPE ? RB : 1;
     const int first = rb;
@@ -525,15 +535,6 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
     // i = 0: (x0, x4), 1: (x1, x5), 2: (x2, x6), 3: (x3, x7) of elements 8 d .. 8 d + 7.
     uint32_t xp[NIT][16];
     float m8sx[NIT];                                    // -8 * sum of the block's activations
-    uint32_t raw[NIT][16];
-    #pragma unroll
-    for (int j = 0; j < NIT; ++j) {
-        if (j * EIT + koff < KT) load_dwords<16, false>(raw[j], x + j * EIT + koff);
-        else {
-            #pragma unroll
-            for (int i = 0; i < 16; ++i) raw[j][i] = 0u;
-        }
-    }
     #pragma unroll
     for (int j = 0; j < NIT; ++j) {
         float sx = 0.0f;
