@@ -152,6 +152,11 @@ def test_smollm_widths_fp16_and_q4_weights_on_device(kind):
     ("wide_heads", dict(hidden=1024, inter=1536, n_heads=8, n_kv_heads=2, head_dim=128, n_layers=2, vocab=2048,
                         max_pos=80, rms_eps=1e-6, rope_theta=500000.0), 72),   # head_dim 128, K = 1024 / 1536
     ("full_cache", dict(SMOL, max_pos=24, n_layers=1), 23),        # up to the last cache row
+    # the attention launch keeps 128 cache rows per LDS tile: a second tile at head_dim 128, a third
+    # at head_dim 64 (with a context length that is no multiple of anything), cache filled to the end
+    ("wide_heads_two_tiles", dict(hidden=1024, inter=1536, n_heads=8, n_kv_heads=2, head_dim=128, n_layers=1,
+                                  vocab=2048, max_pos=141, rms_eps=1e-6, rope_theta=500000.0), 140),
+    ("three_tiles", dict(SMOL, max_pos=267, n_layers=1), 266),
 ])
 def test_device_step_other_geometries(name, cfg, steps):
     """Long sequences, 128-wide heads and a cache filled to its last row: tokens and the last logits
