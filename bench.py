@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the lm_head int8 GEMV kernel, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # (separate counter runs of this script, scaled by what the same counters read for a
 # device-to-device copy of known size; profiles/gemv_int8_lm_head_hbm_traffic.txt).
-LM_HEAD_I8_TRAFFIC_BYTES = 142342700
+LM_HEAD_I8_TRAFFIC_BYTES = 142203900
 
 
 def algo_bytes_i8(N, K):
