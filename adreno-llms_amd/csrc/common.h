@@ -56,7 +56,7 @@ struct GemvCall {
     int         add_mode = 0;         // EPI_ADD: an AddMode
     // Greedy token: every wavefront of the launch also leaves the best (fp16 value, row) of the rows
     // it computed, by the reference's argmax order for num_partials = am_np, in am_v / am_i
-    // [gemv_argmax_slots() entries]; one segment, M = 1, kernels of gemv_takes_norm only.
+    // [gemv_argmax_slots() entries]; one segment, M = 1, calls that gemv_takes_argmax accepts.
     float*      am_v = nullptr;
     int*        am_i = nullptr;
     int         am_np = 0;
@@ -70,6 +70,7 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n);
 bool gemv_takes_norm(WeightKind kind, int K);    // GemvCall::norm_w is supported for this kind and K
 bool gemv_takes_swiglu(WeightKind kind, int K);  // EPI_SWIGLU is supported for this kind and K
 // Candidates a launch with GemvCall::am_v writes (one per wavefront of its grid), and their upper bound.
+bool gemv_takes_argmax(const GemvCall& c);       // GemvCall::am_v is supported for this call (kind, K, M, epilogue)
 int  gemv_argmax_slots(const GemvCall& c);
 constexpr int kGemvArgmaxMaxSlots = 8192;
 bool launch_gate_up_silu(hipStream_t s, WeightKind kind, int N, int K, const void* x,

@@ -722,6 +722,24 @@ int mi_decoder_step(void* dec, void* stream) {
         return 0;
     if (fused) return 1;
     {
+        // weights whose GEMV has no norm in its prologue (Q4) may still take the argmax in its epilogue
+        WeightKind kind = WK_F16;
+        if (!fused_gemv_kind(d->lm_head, c.vocab, Hd, &kind)) return 0;
+        if (!gemv_takes_norm(kind, Hd)) {
+            hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(64), 0, s, d->h, static_cast<const uint16_t*>(d->final_norm), d->xn,
+                               Hd, c.rms_eps);
+            if (!launched()) return 0;
+            if (!linear_argmax(s, c.vocab, Hd, d->xn, d->lm_head, d->logits, nullptr, 0.0f, 32, next, &d->st->token,
+                               &d->st->pos, &fused))
+                return 0;
+            if (fused) return 1;
+            if (!mi_linear(stream, 1, c.vocab, Hd, d->xn, d->lm_head, d->logits)) return 0;
+            if (!mi_argmax_f16(stream, d->logits, c.vocab, 32, next)) return 0;
+            hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->st);
+            return launched() ? 1 : 0;
+        }
+    }
+    {
         const int N1[1] = {c.vocab};
         const void* const W1[1] = {d->lm_head};
         void* const y1[1] = {d->logits};

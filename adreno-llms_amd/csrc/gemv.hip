@@ -466,7 +466,7 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
 //     block scale multiplies the block sum once.
 // 16 lanes still share a row and a wavefront still streams row batches of 4 rows with the
 // same double-buffered fetch; each lane owns one scale block per K-iteration.
-template <int KT, int EPI, bool PIPE, int RB>
+template <int KT, int EPI, bool PIPE, int RB, bool AM = false>
 __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restrict__ x, const SegList L) {
     constexpr int EIT = 512;                            // elements per K-iteration (16 lanes x 32)
     constexpr int NIT = (KT + EIT - 1) / EIT;
@@ -486,6 +486,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
         uint16_t res;
         uint16_t* ybase;    // &y[m][first row of the batch], uniform
         int yoff;           // row inside the batch, -1 when the lane's row is past N
+        int row0;           // first row of the batch inside its segment, uniform
     };
     const uint32_t lane_w = r * ROWB + g * 16, lane_w0 = g * 16;
     auto fetch = [&](Batch& b, int rb) {
@@ -498,6 +499,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
         const uint32_t wo = valid ? lane_w : lane_w0;
         b.ybase = sg.y + static_cast<size_t>(m) * sg.N + row0;
         b.yoff = valid ? r : -1;
+        b.row0 = row0;
         if constexpr (EPI == EPI_ADD) b.res = b.ybase[rr];
         #pragma unroll
         for (int j = 0; j < NIT; ++j) {
@@ -511,7 +513,15 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
     // weights are still on their way.
     const int nw = gridDim.x * kWavesPerBlock;
     int rb = blockIdx.x * kWavesPerBlock + wave;
-    if (rb >= L.nbatch) return;
+    const int wid = rb;
+    const TieRule rule{L.am_chunk};
+    Cand top{kArgmaxNone, 0};                                 // AM: best row so far (lanes with g == 0)
+    if (rb >= L.nbatch) {
+        if constexpr (AM) {
+            if (lane == 0) { L.am_v[wid] = kArgmaxNone; L.am_i[wid] = 0; }
+        }
+        return;
+    }
     uint32_t raw[NIT][16];
     #pragma unroll
     for (int j = 0; j < NIT; ++j) {
@@ -579,7 +589,12 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
         acc = add_from_above<1>(acc);
         if (g == 0 && b.yoff >= 0) {
             const float out = EPI == EPI_ADD ? add_residual(acc, 1.0f, h_f(b.res), false, L.add_mode) : acc;
-            b.ybase[b.yoff] = f_h(out);
+            const uint16_t bits = f_h(out);
+            b.ybase[b.yoff] = bits;
+            if constexpr (AM) {
+                const float v = h_f(bits);
+                if (v > kArgmaxNone) top = rule.best(top, Cand{v, b.row0 + b.yoff});
+            }
         }
     };
 
@@ -607,6 +622,10 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
             rb += step;
             if (rb >= L.nbatch) break;
         }
+    }
+    if constexpr (AM) {
+        const Cand w = rule.best_of_wave(top);
+        if (lane == 0) { L.am_v[wid] = w.v; L.am_i[wid] = w.i; }
     }
 }
 
@@ -913,20 +932,32 @@ bool launch_q4_fast(hipStream_t s, const GemvCall* calls, int n, bool* taken) {
     *taken = true;
     const Plan p = make_plan(calls, n, 4);
     const auto* x = static_cast<const uint16_t*>(calls[0].x);
-#define MI_Q4F(KT)                                                                                   \
+#define MI_Q4F(KT, AM)                                                                               \
     case KT:                                                                                         \
         if (p.pipe) {                                                                                \
             constexpr int kRB = group_size(WK_Q4, KT, 4);                                            \
-            hipLaunchKernelGGL((gemv_q4_fast<KT, EPI, true, kRB>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+            hipLaunchKernelGGL((gemv_q4_fast<KT, EPI, true, kRB, AM>), p.grid, dim3(kBlock), 0, s, x, p.L); \
         } else {                                                                                     \
-            hipLaunchKernelGGL((gemv_q4_fast<KT, EPI, false, 1>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+            hipLaunchKernelGGL((gemv_q4_fast<KT, EPI, false, 1, AM>), p.grid, dim3(kBlock), 0, s, x, p.L); \
         }                                                                                            \
         break;
+    if constexpr (EPI == EPI_STORE) {
+        if (p.L.am_v) {
+            switch (K) {
+                MI_Q4F(576, true)
+                MI_Q4F(896, true)
+                MI_Q4F(1024, true)
+                MI_Q4F(1536, true)
+                default: *taken = false; return true;
+            }
+            return MI_HIP_OK(hipGetLastError());
+        }
+    }
     switch (K) {
-        MI_Q4F(576)
-        MI_Q4F(896)
-        MI_Q4F(1024)
-        MI_Q4F(1536)
+        MI_Q4F(576, false)
+        MI_Q4F(896, false)
+        MI_Q4F(1024, false)
+        MI_Q4F(1536, false)
         default: *taken = false; return true;
     }
 #undef MI_Q4F
@@ -964,6 +995,16 @@ bool check_call(const GemvCall& c) {
 
 }  // namespace
 
+// Kernels that can leave argmax candidates: the ones that keep x in registers (int8, fp16) and the
+// Q4 throughput kernel where launch_gemv_group would take it.
+bool gemv_takes_argmax(const GemvCall& c) {
+    if (c.M != 1 || c.epi != EPI_STORE) return false;
+    if (c.kind == WK_Q4)
+        return !c.norm_w && gemv_mode() == 1 && pick_vl(c.kind, 1, c.N, c.K) == 4 &&
+               (c.K == 576 || c.K == 896 || c.K == 1024 || c.K == 1536);
+    return gemv_takes_norm(c.kind, c.K);
+}
+
 int gemv_argmax_slots(const GemvCall& c) {
     const Plan p = make_plan(&c, 1, pick_vl(c.kind, c.M, c.N, c.K));
     return static_cast<int>(p.grid.x) * kWavesPerBlock;
@@ -995,8 +1036,8 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
         rows += calls[i].N;
     }
     const GemvCall& c = calls[0];
-    if (c.am_v && !(n == 1 && c.M == 1 && c.epi == EPI_STORE && c.am_i && c.am_np > 0 && gemv_takes_norm(c.kind, c.K))) {
-        MI_ERROR_FMT("gemv: the fused argmax takes one segment, M = 1, int8 or fp16 weights and a K kept in registers "
+    if (c.am_v && !(n == 1 && c.am_i && c.am_np > 0 && gemv_takes_argmax(c))) {
+        MI_ERROR_FMT("gemv: the fused argmax takes one segment, M = 1 and a kernel that keeps x in registers "
                      "(kind=%d K=%d)", static_cast<int>(c.kind), c.K);
         return false;
     }

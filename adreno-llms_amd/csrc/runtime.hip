@@ -111,11 +111,11 @@ bool linear_argmax(hipStream_t s, int N, int K, const void* x, const void* W, vo
     Entry e;
     if (!resolve("linear_argmax", W, N, K, &e)) return false;
     void* ws = workspace_of(s);
-    if (!ws || !gemv_takes_norm(e.kind, K)) return true;
     GemvCall c;
     c.x = x; c.W = W; c.scale = e.scale; c.y = logits;
     c.M = 1; c.N = N; c.K = K; c.kind = e.kind; c.epi = EPI_STORE;
     c.norm_w = norm_w; c.norm_eps = norm_eps;
+    if (!ws || !gemv_takes_argmax(c) || (norm_w && !gemv_takes_norm(e.kind, K))) return true;
     static_assert(kGemvArgmaxMaxSlots * 8 <= kWorkspaceBytes, "candidates fit the workspace");
     c.am_v = static_cast<float*>(ws);
     c.am_i = reinterpret_cast<int*>(c.am_v + kGemvArgmaxMaxSlots);

@@ -141,11 +141,12 @@ def test_lm_head_then_argmax_on_device():
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind,N,K", [("int8", 151936, 896), ("fp16", 151936, 896), ("int8", 49152, 576),
                                       ("fp16", 30001, 1536), ("int8", 5000, 4864), ("int8", 300, 1024),
-                                      ("q4", 20000, 896), ("int8", 7000, 640)])
+                                      ("q4", 20000, 896), ("q4", 151936, 896), ("q4", 5000, 576), ("q4", 3000, 1024),
+                                      ("int8", 7000, 640)])
 def test_argmax_inside_the_lm_head_launch(kind, N, K):
-    """Where the GEMV keeps x in registers (int8 and fp16, the K of the model families) its wavefronts
-    leave their best rows and a small launch picks the token from those; other kinds and K read the
-    logits back.  Either way: logits as mi_linear's, token as the oracle's from those logits, with
+    """Where the GEMV keeps x in registers (int8 and fp16 at the K of the model families, Q4 where its
+    throughput kernel runs) its wavefronts leave their best rows and a small launch picks the token
+    from those; other K, and Q4 launches too small for that kernel, read the logits back.  Either way: logits as mi_linear's, token as the oracle's from those logits, with
     thousands of equal maxima (W has 40 distinct rows) and for several chunkings."""
     from helpers import synth_w, synth_x
     assert mil.lib().mi_init(0) == 1
