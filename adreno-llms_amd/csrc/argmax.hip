@@ -107,6 +107,9 @@ __global__ __launch_bounds__(kFinishThreads) void argmax_finish_kernel(const flo
                                                                  int* __restrict__ out2, int* __restrict__ counter) {
     const TieRule rule{(N + num_partials - 1) / num_partials};
     Cand c{kNone, 0};
+    // (the counter is read now so that its round trip does not come after the reduction)
+    int count_now = 0;
+    if (counter && threadIdx.x == 0) count_now = counter[0];
     constexpr int kAhead = 4;
     Cand pre[kAhead];
     #pragma unroll
@@ -135,7 +138,7 @@ __global__ __launch_bounds__(kFinishThreads) void argmax_finish_kernel(const flo
         const int token = c.v > kNone ? c.i : 0;
         out[0] = token;
         if (out2) out2[0] = token;
-        if (counter) counter[0] = counter[0] + 1;
+        if (counter) counter[0] = count_now + 1;
     }
 }
 

@@ -18,9 +18,21 @@ struct Cand {
 
 struct TieRule {
     int chunk;      // elements per chunk: ceil(N / num_partials)
+    double inv;     // 1 / chunk
+    __device__ explicit TieRule(int c) : chunk(c), inv(1.0 / static_cast<double>(c)) {}
     __device__ static unsigned rev6(int a) { return __brev(static_cast<unsigned>(a) & 63u) >> 26; }
+    // a / chunk for a >= 0 without an integer division (two of them per tie were most of the
+    // instructions of a reduction step, and candidates tie often: they are the largest fp16 values
+    // of their wavefronts): the product with the rounded reciprocal is off by one at most, and
+    // the remainder says which way.
+    __device__ int chunk_of(int a) const {
+        int q = static_cast<int>(static_cast<double>(a) * inv);
+        const int r = a - q * chunk;
+        q += r < 0 ? -1 : (r >= chunk ? 1 : 0);
+        return q;
+    }
     __device__ bool before(int a, int b) const {          // a wins a tie against b
-        const int ca = a / chunk, cb = b / chunk;
+        const int ca = chunk_of(a), cb = chunk_of(b);
         if (ca != cb) return (ca & 63) != (cb & 63) ? rev6(ca) < rev6(cb) : ca < cb;
         const int la = (a - ca * chunk) & 63, lb = (b - cb * chunk) & 63;
         if (la != lb) return rev6(la) < rev6(lb);
