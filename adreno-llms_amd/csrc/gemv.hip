@@ -12,8 +12,8 @@
 // iteration (one global_load_dwordx4), 16 lanes cover a row-iteration and a 64-wide
 // wavefront works on 4 rows at once ("a row batch"); VL = 2 and VL = 1 trade load width
 // for more wavefronts when N is small.  Tree steps with s >= VL are cross-lane adds inside
-// the 64/VL-lane group (DPP row shifts), steps with s < VL are adds between a lane's own
-// accumulators.
+// the 64/VL-lane group (v_permlane32_swap / v_permlane16_swap across rows of 16 lanes, DPP
+// row shifts inside one), steps with s < VL are adds between a lane's own accumulators.
 //
 // A lane's K positions do not depend on the row, so in the fixed-K kernels the lane loads
 // its slice of x once into registers and then streams row batches: every byte of W is
@@ -25,7 +25,10 @@
 //
 // Several GEMVs that read the same x and have the same K and weight kind (q/k/v, gate/up)
 // can be given to one launch as "segments": the row batches of all segments form one
-// index space.
+// index space.  A decode step also hangs its small kernels on these launches, each with the
+// arithmetic of the separate kernel it replaces: the RMSNorm of x in the prologue, the
+// residual add or the SwiGLU of a gate / up pair in the epilogue, and the first step of the
+// greedy argmax (every wavefront's best row) behind the lm_head.
 #include "common.h"
 #include <hip/hip_fp16.h>
 #include "device_math.h"
