@@ -207,7 +207,7 @@ def test_q4_gemm_single_rounding_mode_within_its_bound(queue, M, N, K):
 
 
 def test_q4_gemm_tiny_scales_keep_fp16_subnormals(queue):
-    """Weights around 1e-4: the block scales and most products q * scale are fp16 subnormals.
+    """Weights near 1e-4: the block scales and most products q * scale are fp16 subnormals.
     They must enter the sums at full value (nothing flushed to zero on the way to the matrix cores)."""
     M, N, K = 64, 512, 896
     W = (synth_w(1960, N, K).astype(np.float32) * np.float32(0.004)).astype(np.float16)
