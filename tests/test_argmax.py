@@ -81,6 +81,27 @@ def test_oracle_argmax_plain_cases():
     assert O.argmax_f16(x, 1) == 34
 
 
+def test_chunk_index_by_reciprocal_multiply_is_exact():
+    """The device tie rule finds an index's chunk as trunc(double(i) * (1.0 / chunk)), corrected by
+    one where the remainder i - q * chunk falls outside [0, chunk) (argmax_rule.h, chunk_of).  The
+    same IEEE double operations in numpy: equal to i // chunk for every index below 2^31, at the
+    chunk boundaries where a rounded reciprocal could land on the wrong side."""
+    rng = np.random.default_rng(3)
+    chunks = np.unique(np.concatenate([
+        np.array([1, 2, 3, 5, 7, 10, 63, 64, 65, 592, 1520, 4748, 151936, 2**20, 2**30, 2**31 - 1]),
+        rng.integers(1, 2**31 - 1, 2000), rng.integers(1, 70000, 2000)])).astype(np.int64)
+    top = np.int64(2**31 - 1)
+    for c in chunks:
+        k = np.unique(np.concatenate([np.arange(0, 40), rng.integers(0, top // c + 1, 300), [top // c]])).astype(np.int64)
+        idx = np.unique(np.clip(np.concatenate([k * c - 1, k * c, k * c + 1, [top]]), 0, top))
+        inv = np.float64(1.0) / np.float64(c)
+        q = np.trunc(idx.astype(np.float64) * inv).astype(np.int64)
+        r = idx - q * c
+        assert np.all((r >= -c) & (r < 2 * c)), int(c)           # off by one at most
+        q = q + np.where(r < 0, -1, np.where(r >= c, 1, 0))
+        assert np.array_equal(q, idx // c), int(c)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("name,x", cases(), ids=[c[0] for c in cases()])
 def test_device_argmax_matches_oracle(name, x):
