@@ -24,6 +24,7 @@ namespace {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kKT = 64;            // K-tile, elements
 constexpr int kLd = kKT + 8;       // LDS row stride, halves
@@ -684,7 +685,9 @@ __global__ __launch_bounds__(256) void gemm_wide(const uint16_t* __restrict__ X,
         if (m >= M) continue;
         uint16_t* dst = out + static_cast<size_t>(m) * N + ncol;
         if (cols8 && ncol + 7 < N) {
-            *reinterpret_cast<u32x4*>(dst) = v;
+            // streaming store: all blocks of a round write their tiles at about the same time, 20 MB at
+            // M = 2048, N = 4864, and nothing reads them back soon (measured: 25.8 -> 24.2 us there)
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
         } else {
             #pragma unroll
             for (int e = 0; e < 8; ++e)
@@ -714,7 +717,8 @@ __global__ __launch_bounds__(256) void reduce_partials(const float* __restrict__
             s0 = __half2float(__ushort_as_half(scale[n])), s1 = __half2float(__ushort_as_half(scale[n + 1]));
             s2 = __half2float(__ushort_as_half(scale[n + 2])), s3 = __half2float(__ushort_as_half(scale[n + 3]));
         }
-        *reinterpret_cast<uint2*>(out + i4) = uint2{pack_half2(a.x * s0, a.y * s1), pack_half2(a.z * s2, a.w * s3)};
+        __builtin_nontemporal_store(u32x2{pack_half2(a.x * s0, a.y * s1), pack_half2(a.z * s2, a.w * s3)},
+                                    reinterpret_cast<u32x2*>(out + i4));
     } else {
         for (int e = 0; e < 4 && i4 + e < MN; ++e) {
             float a = partial[i4 + e];
