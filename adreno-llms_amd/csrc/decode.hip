@@ -722,10 +722,11 @@ int mi_decoder_step(void* dec, void* stream) {
         return 0;
     if (fused) return 1;
     {
-        // weights whose GEMV has no norm in its prologue (Q4) may still take the argmax in its epilogue
+        // Q4: the throughput GEMV has no norm in its prologue but takes the argmax in its epilogue, and
+        // at the lm_head's size it is the faster one: norm as a launch of its own, then that kernel
         WeightKind kind = WK_F16;
         if (!fused_gemv_kind(d->lm_head, c.vocab, Hd, &kind)) return 0;
-        if (!gemv_takes_norm(kind, Hd)) {
+        if (kind == WK_Q4 || !gemv_takes_norm(kind, Hd)) {
             hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(64), 0, s, d->h, static_cast<const uint16_t*>(d->final_norm), d->xn,
                                Hd, c.rms_eps);
             if (!launched()) return 0;

@@ -318,11 +318,20 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
         }
     }
     [[maybe_unused]] uint32_t nrm[NIT][XD];
-    if constexpr (T::EPV == 4) {
-        if (L.norm_w) {
+    // (Q4: a lane's 8-element pieces are not the norm's 4-element ones, so the sum of squares
+    //  takes its own copy of x in the norm's layout: lane l, elements 4 l + 256 j)
+    constexpr int NJ = T::EPV == 8 ? (KT + 255) / 256 : 1;
+    [[maybe_unused]] uint32_t xsq[NJ][2];
+    if (L.norm_w) {
+        #pragma unroll
+        for (int j = 0; j < NIT; ++j)
+            load_dwords<XD, false>(nrm[j], L.norm_w + (j * EIT + koff < KT ? j * EIT + koff : koff));
+        if constexpr (T::EPV == 8) {
             #pragma unroll
-            for (int j = 0; j < NIT; ++j)
-                load_dwords<XD, false>(nrm[j], L.norm_w + (j * EIT + koff < KT ? j * EIT + koff : koff));
+            for (int j = 0; j < NJ; ++j) {
+                if (256 * j + 4 * lane < KT) load_dwords<2, false>(xsq[j], x + 256 * j + 4 * lane);
+                else xsq[j][0] = xsq[j][1] = 0u;
+            }
         }
     }
     Group g0, g1;
@@ -333,27 +342,46 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     // the squares of elements 4 lane + 256 j, the same tree as the GEMV's, then
     // fp16((x * inv) * w)): the virtual lanes of this kernel own exactly those elements, so every
     // wavefront repeats the sum in the reference's order while its first weights are in flight.
-    if constexpr (T::EPV == 4) {
+    {
         if (L.norm_w) {
-            float part[VL];
-            #pragma unroll
-            for (int v = 0; v < VL; ++v) part[v] = 0.0f;
-            #pragma unroll
-            for (int j = 0; j < NIT; ++j) {
-                if (j * EIT + koff < KT) {
-                    #pragma unroll
-                    for (int v = 0; v < VL; ++v) {
-                        const float v0 = lo_f(xr[j][2 * v]), v1 = hi_f(xr[j][2 * v]);
-                        const float v2 = lo_f(xr[j][2 * v + 1]), v3 = hi_f(xr[j][2 * v + 1]);
+            float total;
+            if constexpr (T::EPV == 4) {
+                float part[VL];
+                #pragma unroll
+                for (int v = 0; v < VL; ++v) part[v] = 0.0f;
+                #pragma unroll
+                for (int j = 0; j < NIT; ++j) {
+                    if (j * EIT + koff < KT) {
+                        #pragma unroll
+                        for (int v = 0; v < VL; ++v) {
+                            const float v0 = lo_f(xr[j][2 * v]), v1 = hi_f(xr[j][2 * v]);
+                            const float v2 = lo_f(xr[j][2 * v + 1]), v3 = hi_f(xr[j][2 * v + 1]);
+                            float d = v0 * v0;
+                            d = fmaf(v1, v1, d);
+                            d = fmaf(v2, v2, d);
+                            d = fmaf(v3, v3, d);
+                            part[v] = part[v] + d;
+                        }
+                    }
+                }
+                total = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(reduce_row<VL>(part))));
+            } else {
+                float part = 0.0f;
+                #pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    if (256 * j + 4 * lane < KT) {
+                        const float v0 = lo_f(xsq[j][0]), v1 = hi_f(xsq[j][0]);
+                        const float v2 = lo_f(xsq[j][1]), v3 = hi_f(xsq[j][1]);
                         float d = v0 * v0;
                         d = fmaf(v1, v1, d);
                         d = fmaf(v2, v2, d);
                         d = fmaf(v3, v3, d);
-                        part[v] = part[v] + d;
+                        part = part + d;
                     }
                 }
+                float one[1] = {part};
+                total = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(reduce_row<1>(one))));
             }
-            const float total = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(reduce_row<VL>(part))));
             // (sqrtf: correctly rounded under -fhip-fp32-correctly-rounded-divide-sqrt, which __fsqrt_rn is not)
             const float inv = __fdiv_rn(1.0f, sqrtf(__fdiv_rn(total, static_cast<float>(KT)) + L.norm_eps));
             #pragma unroll
@@ -388,7 +416,7 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
         // g0 holds row batch rb of the gate matrix (segment 0), g1 the same rows of the up
         // matrix (segment 1); the gate and up values are rounded to fp16 as two GEMVs would
         // store them, then gate[n] = fp16((g * sigmoid(g)) * u)  (QW/kernels/mlp.cl swiglu_inplace)
-        static_assert(!PIPE && KIND != WK_Q4, "one batch pair at a time");
+        static_assert(!PIPE, "one batch pair at a time");
         while (true) {
             const float sg_ = row_sum(g0.b[0]), su_ = row_sum(g1.b[0]);
             if (g == 0 && g0.b[0].yoff >= 0) {
@@ -1013,13 +1041,14 @@ int gemv_argmax_slots(const GemvCall& c) {
     return static_cast<int>(p.grid.x) * kWavesPerBlock;
 }
 
-bool gemv_takes_swiglu(WeightKind kind, int K) {
-    return (kind == WK_I8 || kind == WK_F16) && (K == 576 || K == 896 || K == 1024 || K == 1536);
+bool gemv_takes_swiglu(WeightKind, int K) {
+    return K == 576 || K == 896 || K == 1024 || K == 1536;
 }
 
-// The kernels that keep x in registers, with 4-element virtual lanes.
-bool gemv_takes_norm(WeightKind kind, int K) {
-    return (kind == WK_I8 || kind == WK_F16) && (K == 576 || K == 896 || K == 1024 || K == 1536 || K == 4864);
+// The kernels that keep x in registers (every weight kind; Q4 through the exact kernel, not the
+// throughput one).
+bool gemv_takes_norm(WeightKind, int K) {
+    return K == 576 || K == 896 || K == 1024 || K == 1536 || K == 4864;
 }
 
 bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
@@ -1054,8 +1083,8 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
     const int vl = pick_vl(c.kind, c.M, c.epi == EPI_SWIGLU ? rows / 8 : rows, c.K);
     if (c.epi == EPI_SWIGLU) {
         if (n != 2 || calls[0].N != calls[1].N || c.M != 1 || !gemv_takes_swiglu(c.kind, c.K)) {
-            MI_ERROR_FMT("gemv: the SwiGLU epilogue takes a gate and an up matrix of equal N, M = 1, int8 or fp16 "
-                         "weights and K in {576, 896, 1024, 1536} (n=%d kind=%d K=%d)", n, static_cast<int>(c.kind), c.K);
+            MI_ERROR_FMT("gemv: the SwiGLU epilogue takes a gate and an up matrix of equal N, M = 1 "
+                         "and K in {576, 896, 1024, 1536} (n=%d kind=%d K=%d)", n, static_cast<int>(c.kind), c.K);
             return false;
         }
         if (c.kind == WK_I8) {
@@ -1063,10 +1092,15 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
             if (vl == 2) return launch_swiglu_vl<WK_I8, 2>(s, calls);
             return launch_swiglu_vl<WK_I8, 1>(s, calls);
         }
+        if (c.kind == WK_Q4) {
+            if (vl == 4) return launch_swiglu_vl<WK_Q4, 4>(s, calls);
+            if (vl == 2) return launch_swiglu_vl<WK_Q4, 2>(s, calls);
+            return launch_swiglu_vl<WK_Q4, 1>(s, calls);
+        }
         return vl == 2 ? launch_swiglu_vl<WK_F16, 2>(s, calls) : launch_swiglu_vl<WK_F16, 1>(s, calls);
     }
     const bool add = c.epi == EPI_ADD;
-    if (c.kind == WK_Q4 && vl == 4 && gemv_mode() == 1) {
+    if (c.kind == WK_Q4 && vl == 4 && gemv_mode() == 1 && !c.norm_w) {       // (the throughput kernel has no norm)
         bool taken = false;
         const bool ok = add ? launch_q4_fast<EPI_ADD>(s, calls, n, &taken) : launch_q4_fast<EPI_STORE>(s, calls, n, &taken);
         if (taken) return ok;

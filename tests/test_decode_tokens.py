@@ -125,10 +125,10 @@ def test_qwen_shaped_whole_step_on_device_graph_replay():
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind", ["f16", "q4"])
 def test_smollm_widths_fp16_and_q4_weights_on_device(kind):
-    """The device step with fp16 weights (norm, add and SwiGLU ride in the fp16 GEMV kernels) and with
-    Q4 weights (no fused norm for 8-element lanes: separate norm and SwiGLU launches, add in the
-    epilogue), exact GEMV mode: tokens and last logits equal the CPU harness running the oracle's
-    GEMV of the same kind."""
+    """The device step with fp16 and with Q4 weights (norm, add and SwiGLU ride in the GEMV kernels of
+    either kind; the Q4 kernel sums the squares over its own copy of x in the norm's layout), exact
+    GEMV mode: tokens and last logits equal the CPU harness running the oracle's GEMV of the same
+    kind."""
     assert mil.lib().mi_init(0) == 1
     mil.lib().mi_set_gemv_mode(0)
     try:
