@@ -124,6 +124,29 @@ def test_qwen_shaped_whole_step_on_device_graph_replay():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind", ["f16", "q4"])
+def test_qwen_widths_fp16_and_q4_weights_on_device(kind):
+    """The same at Qwen2.5-0.5B widths (K = 896 with norm and SwiGLU, K = 4864 with the residual add),
+    two layers and a small vocabulary."""
+    assert mil.lib().mi_init(0) == 1
+    mil.lib().mi_set_gemv_mode(0)
+    try:
+        queue = mil.Queue()
+        cfg = dict(QWEN25_05B, n_layers=2, vocab=4096, max_pos=48)
+        m = KindModel(cfg, kind, seed=13)
+        want_logits = np.empty(cfg["vocab"], np.uint16)
+        want, _ = greedy(m, PROMPT[:2], 20, linear_cb=m.oracle_cb(), last_logits=want_logits)
+        gd = GpuDecoder(m, queue)
+        got = gd.greedy(PROMPT[:2], 20)
+        got_logits = gd.logits()
+        gd.close()
+        assert got == want and len(set(got)) > 1
+        assert np.array_equal(got_logits, want_logits)
+    finally:
+        mil.lib().mi_set_gemv_mode(1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["f16", "q4"])
 def test_smollm_widths_fp16_and_q4_weights_on_device(kind):
     """The device step with fp16 and with Q4 weights (norm, add and SwiGLU ride in the GEMV kernels of
     either kind; the Q4 kernel sums the squares over its own copy of x in the norm's layout), exact
