@@ -275,6 +275,37 @@ def main():
             "launches_per_step": 24 * 5 + 3, "positions": f"8..{pos_after - 1}", "launch": "hip_graph"}
         dec.close()
 
+        # the same step with block-32 Q4 weights (the LFM2 bundles' format): norm and SwiGLU ride in the
+        # exact Q4 GEMV, the lm_head takes the throughput kernel with the argmax in its epilogue
+        q4_keep, q4_w = [], dict(dec_w)
+        def make_q4(seed, N, K):
+            ph, sh = mil.quantize_q4(mil.synth_normal_f16(seed, 0.02, (N, K)))
+            pb, sb = mil.Buffer.from_host(ph), mil.Buffer.from_host(sh)
+            assert mil.nnopt_register_q4_weight(pb, sb, N, K)
+            q4_keep.extend([pb, sb])
+            return pb
+        shape_of = {n: (N, K) for n, N, K in LAYER_SHAPES}
+        for j, (key, name) in enumerate((("wq", "q"), ("wk", "k"), ("wv", "v"), ("wo", "o"), ("wgate", "gate"),
+                                         ("wup", "up"), ("wdown", "down"))):
+            q4_w[key] = [make_q4(9000 + l * 16 + j, *shape_of[name]) for l in range(LAYERS)]
+        q4_w["lm_head"] = make_q4(8999, VOCAB, H)
+        dec = mil.Decoder(cfg, q4_w)
+        assert dec.reset(queue, 0, 785)
+        assert dec.step(queue)
+        queue.finish()
+        assert dec.reset(queue, 0, 785)
+        with mil.Graph(queue) as step_graph_q4:
+            assert dec.step(queue)
+        for _ in range(8):
+            step_graph_q4.launch()
+        ms_tok = time_region(mil, queue, step_graph_q4.launch, 64)
+        detail["c4_whole_decode_step_on_device_q4_weights"] = {
+            "us_per_token": round(ms_tok * 1e3, 1), "tokens_per_s": round(1e3 / ms_tok, 1), "launch": "hip_graph"}
+        dec.close()
+        for i in range(0, len(q4_keep), 2):
+            mil.nnopt_unregister_weight(q4_keep[i])
+        del q4_keep, q4_w
+
     # ---- config 5: prefill GEMM with fused int8 dequant on the matrix cores ---------------
     if not args.no_detail:
         MFMA_PEAK_TFLOPS = 2500.0
