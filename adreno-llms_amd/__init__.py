@@ -60,6 +60,7 @@ _SIGNATURES = {
     "mi_decoder_reset": (_i, [_vp, _vp, _i, _i]),
     "mi_decoder_set_token": (_i, [_vp, _vp, _i]),
     "mi_decoder_step": (_i, [_vp, _vp]),
+    "mi_decoder_prefill": (_i, [_vp, _vp, C.POINTER(_i), _i, _i]),
     "mi_decoder_read": (_i, [_vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
     "mi_decoder_logits": (_vp, [_vp]),
     "mi_decoder_buffer": (_vp, [_vp, _i]),
@@ -337,6 +338,11 @@ class Decoder:
 
     def step(self, queue):
         return bool(lib().mi_decoder_step(self.handle, _q(queue)))
+
+    def prefill(self, queue, tokens, pos0=0):
+        """A prompt at once (Model::forward with seq_len = len(tokens), QW/src/model.cpp:243-376)."""
+        arr = (_i * len(tokens))(*[int(t) for t in tokens])
+        return bool(lib().mi_decoder_prefill(self.handle, _q(queue), arr, len(tokens), pos0))
 
     def read(self, queue):
         pos, tok = _i(), _i()

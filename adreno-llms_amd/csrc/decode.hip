@@ -59,6 +59,8 @@ __global__ __launch_bounds__(64) void rmsnorm_kernel(const uint16_t* __restrict_
     // (cols <= 256 kGroups); the tail that is not a whole group, and longer rows, go through memory.
     constexpr int kGroups = 8;
     const int lid = threadIdx.x, c4n = cols >> 2;
+    x += static_cast<size_t>(blockIdx.x) * cols;       // block b takes row b (a prompt's rows; one row in a decode step)
+    out += static_cast<size_t>(blockIdx.x) * cols;
     typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
     u16x4 xv[kGroups], wv[kGroups];
     float acc = 0.0f;
@@ -447,6 +449,145 @@ __global__ void swiglu_kernel(uint16_t* __restrict__ gate, const uint16_t* __res
     }
 }
 
+
+// ---- a prompt of M tokens at once (Model::forward with seq_len = M, QW/src/model.cpp:243-376) ----
+// Row r of every buffer belongs to position pos0 + r.  The kernels below repeat, row by row, the
+// operations of the single-token kernels above in the same order, so that a prompt gives the
+// same cache rows and logits as M single-token steps wherever the projections do (they do bit
+// for bit when the M > 1 projections run as rows of GEMV, and within the GEMM's tolerance when
+// they run on the matrix cores).
+
+// H[r][c] = embed[tokens[r]][c]   (QW/kernels/embedding.cl)
+__global__ void embed_rows_kernel(const uint16_t* __restrict__ embed, const int* __restrict__ tokens,
+                                  uint16_t* __restrict__ H, int hidden, int vocab) {
+    int t = tokens[blockIdx.x];
+    t = t < 0 ? 0 : (t >= vocab ? vocab - 1 : t);
+    const uint16_t* src = embed + static_cast<size_t>(t) * hidden;
+    uint16_t* dst = H + static_cast<size_t>(blockIdx.x) * hidden;
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = src[c];
+}
+
+// One block per row: q/k/v bias, rotary embedding of q and k at position pos0 + row, k and v into
+// the cache rows of that position (QW/kernels/bias_add.cl, rope.cl; rows as QW/src/layers/
+// attention.cpp:560-600).
+__global__ __launch_bounds__(256) void rope_rows_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ Kp,
+                                                        const uint16_t* __restrict__ V, const uint16_t* __restrict__ bq,
+                                                        const uint16_t* __restrict__ bk, const uint16_t* __restrict__ bv,
+                                                        const uint16_t* __restrict__ cosT, const uint16_t* __restrict__ sinT,
+                                                        uint16_t* __restrict__ kc, uint16_t* __restrict__ vc,
+                                                        uint16_t* __restrict__ QR, int pos0, int n_heads, int n_kv_heads, int D) {
+    const int row = blockIdx.x, pos = pos0 + row, hd2 = D / 2, qd = n_heads * D, kvd = n_kv_heads * D;
+    const uint16_t* cr = cosT + static_cast<size_t>(pos) * D;
+    const uint16_t* sr = sinT + static_cast<size_t>(pos) * D;
+    for (int j = threadIdx.x; j < (n_heads + n_kv_heads) * hd2; j += blockDim.x) {
+        const int head = j / hd2, i = j - head * hd2;
+        const bool isq = head < n_heads;
+        const int hh = isq ? head : head - n_heads;
+        const uint16_t* buf = isq ? Q + static_cast<size_t>(row) * qd + hh * D : Kp + static_cast<size_t>(row) * kvd + hh * D;
+        const uint16_t* bias = (isq ? bq : bk) + hh * D;
+        uint16_t* dst = isq ? QR + static_cast<size_t>(row) * qd + hh * D : kc + static_cast<size_t>(pos) * kvd + hh * D;
+        const float c = h_f(cr[i]), sn = h_f(sr[i]);
+        const float x1 = h_f(f_h(h_f(buf[i]) + h_f(bias[i])));
+        const float x2 = h_f(f_h(h_f(buf[i + hd2]) + h_f(bias[i + hd2])));
+        dst[i] = f_h(fmaf(x1, c, -(x2 * sn)));
+        dst[i + hd2] = f_h(fmaf(x2, c, x1 * sn));
+    }
+    for (int e = threadIdx.x; e < kvd; e += blockDim.x)
+        vc[static_cast<size_t>(pos) * kvd + e] = f_h(h_f(V[static_cast<size_t>(row) * kvd + e]) + h_f(bv[e]));
+}
+
+// One block per (query head, row): the query of position pos0 + row against cache rows
+// 0 .. pos0 + row (causal), QW/kernels/attention.cl gqa_attn_scores, gqa_softmax, gqa_attn_out with
+// the sums in the order of rope_attention_kernel.  Dynamic LDS: 2 D bytes + 6 bytes per position.
+__global__ __launch_bounds__(256) void attention_rows_kernel(const uint16_t* __restrict__ QR, const uint16_t* __restrict__ kc,
+                                                             const uint16_t* __restrict__ vc, uint16_t* __restrict__ out,
+                                                             int pos0, int seq_cap, int n_heads, int n_kv_heads, int D,
+                                                             float scale) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t qv[];
+    float* ex = reinterpret_cast<float*>(qv + D);
+    uint16_t* sc = reinterpret_cast<uint16_t*>(ex + seq_cap);
+    __shared__ float red[64];
+    __shared__ float inv_s;
+    const int qh = blockIdx.x, row = blockIdx.y, pos = pos0 + row, seq_k = pos + 1;
+    const int nrep = n_heads / n_kv_heads, kvh = qh / nrep, kvd = n_kv_heads * D, qd = n_heads * D;
+    const int tid = threadIdx.x, nt = blockDim.x;
+    for (int i = tid; i < D; i += nt) qv[i] = QR[static_cast<size_t>(row) * qd + qh * D + i];
+    __syncthreads();
+    for (int tk = tid; tk < seq_k; tk += nt) {
+        typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+        const u16x4* kv = reinterpret_cast<const u16x4*>(kc + static_cast<size_t>(tk) * kvd + kvh * D);
+        const u16x4* qq = reinterpret_cast<const u16x4*>(qv);
+        float acc = 0.0f;
+        for (int d4 = 0; d4 < D / 4; ++d4) {
+            const u16x4 a = qq[d4], b = kv[d4];
+            float t = h_f(a[0]) * h_f(b[0]);
+            t = fmaf(h_f(a[1]), h_f(b[1]), t);
+            t = fmaf(h_f(a[2]), h_f(b[2]), t);
+            t = fmaf(h_f(a[3]), h_f(b[3]), t);
+            acc = acc + t;
+        }
+        sc[tk] = f_h(acc * scale);
+    }
+    __syncthreads();
+    float m = -3.402823466e+38f;
+    for (int c = tid; c < seq_k; c += nt) m = fmaxf(m, h_f(sc[c]));
+    if (tid < 64) red[tid] = -3.402823466e+38f;
+    __syncthreads();
+    for (int s = 32; s > 0; s >>= 1) m = fmaxf(m, __shfl_down(m, s, 64));
+    if ((tid & 63) == 0) red[tid >> 6] = m;
+    __syncthreads();
+    float maxv = red[0];
+    for (int i = 1; i < (nt + 63) / 64; ++i) maxv = fmaxf(maxv, red[i]);
+    for (int c = tid; c < seq_k; c += nt) {
+        const float e = exp_poly(h_f(sc[c]) - maxv);
+        ex[c] = e;
+        sc[c] = f_h(e);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        float sum = 0.0f;
+        for (int c = 0; c < seq_k; ++c) sum = sum + ex[c];
+        inv_s = rcp_rn(sum + 1e-20f);
+    }
+    __syncthreads();
+    const float inv = inv_s;
+    for (int c = tid; c < seq_k; c += nt) sc[c] = f_h(h_f(sc[c]) * inv);
+    __syncthreads();
+    for (int e = tid; e < D; e += nt) {
+        const uint16_t* col = vc + kvh * D + e;
+        float acc = 0.0f;
+        int tk = 0;
+        for (; tk + 8 <= seq_k; tk += 8) {
+            uint16_t v[8];
+            #pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = col[static_cast<size_t>(tk + u) * kvd];
+            #pragma unroll
+            for (int u = 0; u < 8; ++u) acc = fmaf(h_f(sc[tk + u]), h_f(v[u]), acc);
+        }
+        for (; tk < seq_k; ++tk) acc = fmaf(h_f(sc[tk]), h_f(col[static_cast<size_t>(tk) * kvd]), acc);
+        out[static_cast<size_t>(row) * qd + qh * D + e] = f_h(acc);
+    }
+}
+
+// H[i] = fp16(H[i] + T[i]): the element-wise add behind a projection (QW/kernels/utils.cl element_add)
+__global__ void add_rows_kernel(uint16_t* __restrict__ H, const uint16_t* __restrict__ T, long n) {
+    for (long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += static_cast<long>(gridDim.x) * blockDim.x)
+        H[i] = f_h(h_f(T[i]) + h_f(H[i]));
+}
+
+// gate[i] = swiglu(gate[i], up[i]) over any number of elements (swiglu_kernel takes an int count)
+__global__ void swiglu_rows_kernel(uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, long n) {
+    for (long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += static_cast<long>(gridDim.x) * blockDim.x) {
+        const float g = h_f(gate[i]), u = h_f(up[i]);
+        const float sig = rcp_rn(1.0f + exp_poly(-g));
+        gate[i] = f_h((g * sig) * u);
+    }
+}
+
+// the state a prompt leaves behind for the launches that pick the next token: they read the
+// last prompt position and advance it
+__global__ void set_pos_kernel(State* st, int pos) { st->pos = pos; }
+
 // Dynamic LDS of rope_attention_tiled<D>.
 inline size_t tiled_attention_lds(int D, int max_pos) {
     const size_t head = (static_cast<size_t>(3 * D + 3 * max_pos + 7) & ~static_cast<size_t>(7)) * 2;
@@ -472,6 +613,10 @@ struct Decoder {
     uint16_t *gate = nullptr, *up = nullptr, *logits = nullptr;
     State* st = nullptr;
     std::vector<void*> owned;
+    // rows of a prompt (mi_decoder_prefill): one allocation, made on the first prompt and again
+    // only for a longer one
+    void* prompt_mem = nullptr;
+    int prompt_rows = 0;
 };
 
 template <typename T>
@@ -571,6 +716,7 @@ int mi_decoder_destroy(void* dec) {
     auto* d = static_cast<Decoder*>(dec);
     if (!d) return 1;
     for (void* p : d->owned) (void)hipFree(p);
+    if (d->prompt_mem) (void)hipFree(d->prompt_mem);
     delete d;
     return 1;
 }
@@ -625,6 +771,51 @@ const void* mi_decoder_buffer(void* dec, int which) {
         case 7: return d->sinT;
         default: return nullptr;
     }
+}
+
+// The end of a step and of a prompt: final norm, lm_head, greedy token; the token moves into the
+// device state and the position advances.  d->h holds the residual stream of the last position.
+static int decoder_pick_next(Decoder* d, void* stream) {
+    const mi_decoder_config& c = d->c;
+    auto s = static_cast<hipStream_t>(stream);
+    const int Hd = c.hidden;
+    auto launched = [] { return MI_HIP_OK(hipGetLastError()); };
+    // (the fused argmax's second launch also does what advance_kernel does)
+    void* next = reinterpret_cast<char*>(d->st) + offsetof(State, next);
+    bool fused = false;
+    if (!linear_argmax(s, c.vocab, Hd, d->h, d->lm_head, d->logits, d->final_norm, c.rms_eps, 32, next, &d->st->token,
+                       &d->st->pos, &fused))
+        return 0;
+    if (fused) return 1;
+    {
+        // Q4: the throughput GEMV has no norm in its prologue but takes the argmax in its epilogue, and
+        // at the lm_head's size it is the faster one: norm as a launch of its own, then that kernel
+        WeightKind kind = WK_F16;
+        if (!fused_gemv_kind(d->lm_head, c.vocab, Hd, &kind)) return 0;
+        if (kind == WK_Q4 || !gemv_takes_norm(kind, Hd)) {
+            hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(64), 0, s, d->h, static_cast<const uint16_t*>(d->final_norm), d->xn,
+                               Hd, c.rms_eps);
+            if (!launched()) return 0;
+            if (!linear_argmax(s, c.vocab, Hd, d->xn, d->lm_head, d->logits, nullptr, 0.0f, 32, next, &d->st->token,
+                               &d->st->pos, &fused))
+                return 0;
+            if (fused) return 1;
+            if (!mi_linear(stream, 1, c.vocab, Hd, d->xn, d->lm_head, d->logits)) return 0;
+            if (!mi_argmax_f16(stream, d->logits, c.vocab, 32, next)) return 0;
+            hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->st);
+            return launched() ? 1 : 0;
+        }
+    }
+    {
+        // the head's GEMV takes the norm in its prologue (checked above) but not the argmax in its epilogue
+        const int N1[1] = {c.vocab};
+        const void* const W1[1] = {d->lm_head};
+        void* const y1[1] = {d->logits};
+        if (!fused_gemv(s, 1, N1, Hd, d->h, W1, y1, d->final_norm, c.rms_eps, EPI_STORE)) return 0;
+        if (!mi_argmax_f16(stream, d->logits, c.vocab, 32, next)) return 0;
+    }
+    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->st);
+    return launched() ? 1 : 0;
 }
 
 int mi_decoder_step(void* dec, void* stream) {
@@ -714,41 +905,104 @@ int mi_decoder_step(void* dec, void* stream) {
         }
         if (!linear_into_h(c.inter, d->gate, d->wdown[l])) return 0;
     }
-    // (the fused argmax's second launch also does what advance_kernel does)
-    void* next = reinterpret_cast<char*>(d->st) + offsetof(State, next);
-    bool fused = false;
-    if (!linear_argmax(s, c.vocab, Hd, d->h, d->lm_head, d->logits, d->final_norm, c.rms_eps, 32, next, &d->st->token,
-                       &d->st->pos, &fused))
-        return 0;
-    if (fused) return 1;
-    {
-        // Q4: the throughput GEMV has no norm in its prologue but takes the argmax in its epilogue, and
-        // at the lm_head's size it is the faster one: norm as a launch of its own, then that kernel
-        WeightKind kind = WK_F16;
-        if (!fused_gemv_kind(d->lm_head, c.vocab, Hd, &kind)) return 0;
-        if (kind == WK_Q4 || !gemv_takes_norm(kind, Hd)) {
-            hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(64), 0, s, d->h, static_cast<const uint16_t*>(d->final_norm), d->xn,
-                               Hd, c.rms_eps);
-            if (!launched()) return 0;
-            if (!linear_argmax(s, c.vocab, Hd, d->xn, d->lm_head, d->logits, nullptr, 0.0f, 32, next, &d->st->token,
-                               &d->st->pos, &fused))
-                return 0;
-            if (fused) return 1;
-            if (!mi_linear(stream, 1, c.vocab, Hd, d->xn, d->lm_head, d->logits)) return 0;
-            if (!mi_argmax_f16(stream, d->logits, c.vocab, 32, next)) return 0;
-            hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->st);
-            return launched() ? 1 : 0;
-        }
-    }
-    {
-        const int N1[1] = {c.vocab};
-        const void* const W1[1] = {d->lm_head};
-        void* const y1[1] = {d->logits};
-        if (!norm_linear(d->final_norm, 1, N1, W1, y1, false)) return 0;
-        if (!mi_argmax_f16(stream, d->logits, c.vocab, 32, next)) return 0;
-    }
-    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->st);
-    return launched() ? 1 : 0;
+    return decoder_pick_next(d, stream);
 }
+
+int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens, int pos0) {
+    auto* d = static_cast<Decoder*>(dec);
+    if (!d || !tokens || n_tokens < 1 || pos0 < 0 || static_cast<long>(pos0) + n_tokens > d->c.max_pos) {
+        MI_ERROR_FMT("mi_decoder_prefill: bad argument (n_tokens=%d pos0=%d, max_pos=%d)", n_tokens, pos0,
+                     d ? d->c.max_pos : 0);
+        return 0;
+    }
+    const mi_decoder_config& c = d->c;
+    auto s = static_cast<hipStream_t>(stream);
+    const int M = n_tokens, Hd = c.hidden, D = c.head_dim, qd = c.n_heads * D, kvd = c.n_kv_heads * D, I = c.inter;
+    const float scale = 1.0f / sqrtf(static_cast<float>(D));
+    auto launched = [] { return MI_HIP_OK(hipGetLastError()); };
+
+    // rows of the prompt: H, XN, T [M, hidden]; Q, QR, ATT [M, qd]; K, V [M, kvd]; G, U [M, inter]; tokens
+    const size_t row_halves = 3 * static_cast<size_t>(Hd) + 3 * static_cast<size_t>(qd) + 2 * static_cast<size_t>(kvd) +
+                              2 * static_cast<size_t>(I);
+    if (M > d->prompt_rows) {
+        if (d->prompt_mem) {
+            if (!MI_HIP_OK(hipStreamSynchronize(s))) return 0;      // an earlier prompt may still be running in it
+            (void)hipFree(d->prompt_mem);
+            d->prompt_mem = nullptr;
+            d->prompt_rows = 0;
+        }
+        // every block starts at a multiple of 16 bytes: the row counts are padded to 8 halves per block
+        const size_t bytes = (row_halves * M + 10 * 8) * 2 + static_cast<size_t>(M) * 4 + 16;
+        if (!MI_HIP_OK(hipMalloc(&d->prompt_mem, bytes))) {
+            d->prompt_mem = nullptr;
+            return 0;
+        }
+        d->prompt_rows = M;
+    }
+    const int cap = d->prompt_rows;
+    auto* base = static_cast<uint16_t*>(d->prompt_mem);
+    size_t at = 0;
+    auto carve = [&](size_t halves_per_row) {
+        uint16_t* p = base + at;
+        at += (halves_per_row * cap + 7) & ~static_cast<size_t>(7);
+        return p;
+    };
+    uint16_t *H = carve(Hd), *XN = carve(Hd), *T = carve(Hd), *Q = carve(qd), *QR = carve(qd), *ATT = carve(qd);
+    uint16_t *Kp = carve(kvd), *V = carve(kvd), *G = carve(I), *U = carve(I);
+    int* tok = reinterpret_cast<int*>(base + at);
+
+    if (!MI_HIP_OK(hipMemcpyAsync(tok, tokens, static_cast<size_t>(M) * 4, hipMemcpyHostToDevice, s))) return 0;
+    hipLaunchKernelGGL(embed_rows_kernel, dim3(M), dim3(256), 0, s, static_cast<const uint16_t*>(d->embed), tok, H, Hd, c.vocab);
+    if (!launched()) return 0;
+    const long nH = static_cast<long>(M) * Hd, nI = static_cast<long>(M) * I;
+    const unsigned gH = static_cast<unsigned>(nH / 256 + 1 < 4096 ? nH / 256 + 1 : 4096);
+    const unsigned gI = static_cast<unsigned>(nI / 256 + 1 < 8192 ? nI / 256 + 1 : 8192);
+    const size_t att_lds = static_cast<size_t>(D) * 2 + static_cast<size_t>(pos0 + M) * 6;
+    if (att_lds > 65536) {
+        static bool raised = false;
+        if (!raised && !MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_rows_kernel),
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                      D * 2 + kMaxPositions * 6)))
+            return 0;
+        raised = true;
+    }
+    for (int l = 0; l < c.n_layers; ++l) {
+        hipLaunchKernelGGL(rmsnorm_kernel, dim3(M), dim3(64), 0, s, H, static_cast<const uint16_t*>(d->in_norm[l]), XN, Hd,
+                           c.rms_eps);
+        if (!launched()) return 0;
+        if (!mi_linear(stream, M, qd, Hd, XN, d->wq[l], Q) || !mi_linear(stream, M, kvd, Hd, XN, d->wk[l], Kp) ||
+            !mi_linear(stream, M, kvd, Hd, XN, d->wv[l], V))
+            return 0;
+        uint16_t* kc = d->kc + static_cast<size_t>(l) * c.max_pos * kvd;
+        uint16_t* vc = d->vc + static_cast<size_t>(l) * c.max_pos * kvd;
+        hipLaunchKernelGGL(rope_rows_kernel, dim3(M), dim3(256), 0, s, Q, Kp, V, static_cast<const uint16_t*>(d->bq[l]),
+                           static_cast<const uint16_t*>(d->bk[l]), static_cast<const uint16_t*>(d->bv[l]), d->cosT, d->sinT,
+                           kc, vc, QR, pos0, c.n_heads, c.n_kv_heads, D);
+        if (!launched()) return 0;
+        hipLaunchKernelGGL(attention_rows_kernel, dim3(c.n_heads, M), dim3(256), att_lds, s, QR, kc, vc, ATT, pos0, pos0 + M,
+                           c.n_heads, c.n_kv_heads, D, scale);
+        if (!launched()) return 0;
+        if (!mi_linear(stream, M, Hd, qd, ATT, d->wo[l], T)) return 0;
+        hipLaunchKernelGGL(add_rows_kernel, dim3(gH), dim3(256), 0, s, H, T, nH);
+        if (!launched()) return 0;
+        hipLaunchKernelGGL(rmsnorm_kernel, dim3(M), dim3(64), 0, s, H, static_cast<const uint16_t*>(d->post_norm[l]), XN, Hd,
+                           c.rms_eps);
+        if (!launched()) return 0;
+        if (!mi_linear(stream, M, I, Hd, XN, d->wgate[l], G) || !mi_linear(stream, M, I, Hd, XN, d->wup[l], U)) return 0;
+        hipLaunchKernelGGL(swiglu_rows_kernel, dim3(gI), dim3(256), 0, s, G, U, nI);
+        if (!launched()) return 0;
+        if (!mi_linear(stream, M, Hd, I, G, d->wdown[l], T)) return 0;
+        hipLaunchKernelGGL(add_rows_kernel, dim3(gH), dim3(256), 0, s, H, T, nH);
+        if (!launched()) return 0;
+    }
+    // only the last position picks a token: its residual stream becomes the single-token state
+    if (!MI_HIP_OK(hipMemcpyAsync(d->h, H + static_cast<size_t>(M - 1) * Hd, static_cast<size_t>(Hd) * 2,
+                                  hipMemcpyDeviceToDevice, s)))
+        return 0;
+    hipLaunchKernelGGL(set_pos_kernel, dim3(1), dim3(1), 0, s, d->st, pos0 + M - 1);
+    if (!launched()) return 0;
+    return decoder_pick_next(d, stream);
+}
+
 
 }  // extern "C"

@@ -64,6 +64,20 @@ int   mi_decoder_set_token(void* decoder, void* stream, int token);
  * last valid one (later steps clamp the position and overwrite that row). */
 int   mi_decoder_step(void* decoder, void* stream);
 
+/* A prompt at once: Model::forward with seq_len = n_tokens (QW/src/model.cpp:243-376), where every
+ * pytorch_linear is an M = n_tokens call (QW/src/utils.cpp:785-796) and so reaches the GEMM of
+ * mi_linear.  Consumes tokens[0 .. n_tokens) (host memory) at positions pos0 .. pos0 + n_tokens - 1,
+ * writes their KV rows (rows below pos0 are read as they are), leaves the greedy token after the
+ * last one as the device token and pos0 + n_tokens as the device position: the state n_tokens
+ * calls of mi_decoder_step with the tokens forced would leave.  The cache rows and the logits
+ * are those of such steps bit for bit when the M > 1 projections run as rows of GEMV
+ * (mi_set_gemm_mode(1), the reference's quantised prefill, LF/src/model.cpp:243-250), and within
+ * the GEMM's tolerance of them on the matrix cores.  pos0 + n_tokens <= max_pos.  The first prompt,
+ * and any longer one later, allocates the prompt's activation rows (about 31 KB per token at
+ * Qwen2.5-0.5B widths); not for graph capture.  mi_decoder_buffer(0) afterwards holds the residual
+ * stream of the last position; buffers 1 .. 5 are left as they were. */
+int   mi_decoder_prefill(void* decoder, void* stream, const int* tokens, int n_tokens, int pos0);
+
 /* Reads the device state back (synchronises the stream). */
 int   mi_decoder_read(void* decoder, void* stream, int* pos, int* token);
 /* fp16 [vocab] logits of the last step, in device memory. */
