@@ -498,13 +498,16 @@ __global__ __launch_bounds__(256) void rope_rows_kernel(const uint16_t* __restri
 
 // One block per (query head, row): the query of position pos0 + row against cache rows
 // 0 .. pos0 + row (causal), QW/kernels/attention.cl gqa_attn_scores, gqa_softmax, gqa_attn_out with
-// the sums in the order of rope_attention_kernel.  Dynamic LDS: 2 D bytes + 6 bytes per position.
+// the sums in the order of rope_attention_kernel.  256 threads.  Dynamic LDS: 2 D (1 + kPromptTile)
+// bytes + 6 bytes per position.
+constexpr int kPromptTile = 64;
 __global__ __launch_bounds__(256) void attention_rows_kernel(const uint16_t* __restrict__ QR, const uint16_t* __restrict__ kc,
                                                              const uint16_t* __restrict__ vc, uint16_t* __restrict__ out,
                                                              int pos0, int seq_cap, int n_heads, int n_kv_heads, int D,
                                                              float scale) {
     extern __shared__ __attribute__((aligned(16))) uint16_t qv[];
-    float* ex = reinterpret_cast<float*>(qv + D);
+    uint16_t* tile = qv + D;                                       // [kPromptTile][D] values
+    float* ex = reinterpret_cast<float*>(tile + kPromptTile * D);
     uint16_t* sc = reinterpret_cast<uint16_t*>(ex + seq_cap);
     __shared__ float red[64];
     __shared__ float inv_s;
@@ -553,20 +556,225 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(const uint16_t* __r
     const float inv = inv_s;
     for (int c = tid; c < seq_k; c += nt) sc[c] = f_h(h_f(sc[c]) * inv);
     __syncthreads();
-    for (int e = tid; e < D; e += nt) {
-        const uint16_t* col = vc + kvh * D + e;
-        float acc = 0.0f;
-        int tk = 0;
-        for (; tk + 8 <= seq_k; tk += 8) {
-            uint16_t v[8];
-            #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = col[static_cast<size_t>(tk + u) * kvd];
-            #pragma unroll
-            for (int u = 0; u < 8; ++u) acc = fmaf(h_f(sc[tk + u]), h_f(v[u]), acc);
+    // values: tiles of kPromptTile cache rows go through LDS (all threads fetch, 8 bytes each), then
+    // thread e < D runs its sum over the tile's keys in index order
+    typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+    u16x4* tile4 = reinterpret_cast<u16x4*>(tile);
+    const int d4n = D / 4;
+    float acc = 0.0f;                                   // of output element tid (D <= 256 = threads)
+    for (int t0 = 0; t0 < seq_k; t0 += kPromptTile) {
+        const int rows = seq_k - t0 < kPromptTile ? seq_k - t0 : kPromptTile;
+        for (int i = tid; i < rows * d4n; i += nt) {
+            const int r = i / d4n, p = i - r * d4n;
+            tile4[i] = *reinterpret_cast<const u16x4*>(vc + static_cast<size_t>(t0 + r) * kvd + kvh * D + 4 * p);
         }
-        for (; tk < seq_k; ++tk) acc = fmaf(h_f(sc[tk]), h_f(col[static_cast<size_t>(tk) * kvd]), acc);
-        out[static_cast<size_t>(row) * qd + qh * D + e] = f_h(acc);
+        __syncthreads();
+        if (tid < D)
+            for (int r = 0; r < rows; ++r) acc = fmaf(h_f(sc[t0 + r]), h_f(tile[r * D + tid]), acc);
+        __syncthreads();
     }
+    if (tid < D) out[static_cast<size_t>(row) * qd + qh * D + tid] = f_h(acc);
+}
+
+// The same for head widths 64 and 128 with at most 8 query heads per key/value head: one block per
+// (key/value head, row) serves all query heads of the group, so that a cache row is fetched once
+// per group and position instead of once per head, and every fetch is a coalesced copy of a tile
+// of kPromptTile rows into LDS (a thread of attention_rows_kernel walks a cache row of its own,
+// which the memory pipeline serves one line per thread).  Per query the operations and their
+// order are those of attention_rows_kernel: a score per thread from the key tile (rows padded by
+// 8 bytes against bank conflicts), maximum, exponentials, the denominator summed by one thread
+// in key order, the output element's sum in key order from the value tiles.  A (query, key)
+// pair owns 4 bytes of LDS that hold, in turn, its fp16 score, its fp32 exponential and its fp16
+// probability.  Wavefront w serves queries w and w + 4 in every phase but the last, where a thread
+// owns one output element of up to 8 D / 256 queries.
+// Dynamic LDS: 16 D + 2 kPromptTile (D + 4) + 4 nrep seq_cap bytes; seq_cap is a multiple of 4.
+template <int D>
+__global__ __launch_bounds__(256) void attention_group_kernel(const uint16_t* __restrict__ QR, const uint16_t* __restrict__ kc,
+                                                              const uint16_t* __restrict__ vc, uint16_t* __restrict__ out,
+                                                              int pos0, int seq_cap, int n_heads, int n_kv_heads, float scale) {
+    typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+    constexpr int TK = kPromptTile, KS = D + 4, D4 = D / 4;
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+    uint16_t* qv = smem;                                            // [8][D]
+    uint16_t* tile = qv + 8 * D;                                    // [TK][KS] keys, then [TK][D] values
+    uint32_t* slot = reinterpret_cast<uint32_t*>(tile + TK * KS);   // [nrep][seq_cap]
+    __shared__ float inv_s[8];
+    const int g = blockIdx.x, row = blockIdx.y, pos = pos0 + row, seq_k = pos + 1;
+    const int nrep = n_heads / n_kv_heads, kvd = n_kv_heads * D, qd = n_heads * D;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const uint16_t* qsrc = QR + static_cast<size_t>(row) * qd + static_cast<size_t>(g) * nrep * D;   // the group's heads are adjacent
+    for (int i = tid; i < nrep * D; i += 256) qv[i] = qsrc[i];
+    const bool has0 = w < nrep, has1 = w + 4 < nrep;
+    const int q0i = has0 ? w : 0, q1i = has1 ? w + 4 : q0i;
+
+    // A tile's rows travel global memory -> registers -> LDS; the next tile's are requested before
+    // the current tile is worked on, so that their latency runs under the arithmetic.
+    constexpr int kPieces = TK * D4 / 256;                          // 8-byte pieces of a tile per thread
+    u16x4 pre[kPieces];
+    auto fetch = [&](const uint16_t* cache, int t0) {
+        #pragma unroll
+        for (int u = 0; u < kPieces; ++u) {
+            const int i = tid + 256 * u, r = i / D4, p = i - r * D4;
+            const int tk = t0 + r < seq_k ? t0 + r : seq_k - 1;     // rows past the last key: a copy of it, never used
+            pre[u] = *reinterpret_cast<const u16x4*>(cache + static_cast<size_t>(tk) * kvd + g * D + 4 * p);
+        }
+    };
+    auto stash = [&](int stride) {
+        #pragma unroll
+        for (int u = 0; u < kPieces; ++u) {
+            const int i = tid + 256 * u, r = i / D4, p = i - r * D4;
+            *reinterpret_cast<u16x4*>(tile + r * stride + 4 * p) = pre[u];
+        }
+    };
+
+    // scores: thread (key = lane, wavefront w) of a tile takes queries w and w + 4
+    fetch(kc, 0);
+    for (int t0 = 0; t0 < seq_k; t0 += TK) {
+        const int rows = seq_k - t0 < TK ? seq_k - t0 : TK;
+        __syncthreads();                                             // q is in place; the last tile has been used
+        stash(KS);
+        __syncthreads();
+        if (t0 + TK < seq_k) fetch(kc, t0 + TK);
+        if (lane < rows) {
+            const u16x4* kr = reinterpret_cast<const u16x4*>(tile + lane * KS);
+            const u16x4* qa = reinterpret_cast<const u16x4*>(qv + q0i * D);
+            const u16x4* qb = reinterpret_cast<const u16x4*>(qv + q1i * D);
+            float acc0 = 0.0f, acc1 = 0.0f;
+            #pragma unroll 8
+            for (int d4 = 0; d4 < D4; ++d4) {
+                const u16x4 b = kr[d4], a0 = qa[d4], a1 = qb[d4];
+                float t = h_f(a0[0]) * h_f(b[0]);
+                t = fmaf(h_f(a0[1]), h_f(b[1]), t);
+                t = fmaf(h_f(a0[2]), h_f(b[2]), t);
+                t = fmaf(h_f(a0[3]), h_f(b[3]), t);
+                acc0 = acc0 + t;
+                float u = h_f(a1[0]) * h_f(b[0]);
+                u = fmaf(h_f(a1[1]), h_f(b[1]), u);
+                u = fmaf(h_f(a1[2]), h_f(b[2]), u);
+                u = fmaf(h_f(a1[3]), h_f(b[3]), u);
+                acc1 = acc1 + u;
+            }
+            if (has0) slot[q0i * seq_cap + t0 + lane] = f_h(acc0 * scale);
+            if (has1) slot[q1i * seq_cap + t0 + lane] = f_h(acc1 * scale);
+        }
+    }
+    fetch(vc, 0);                                                    // the first tile of values arrives under the softmax
+    __syncthreads();
+    // maximum and exponentials, a wavefront per query.  A lane takes four of its entries at a time
+    // (all reads ahead of the arithmetic and the writes: one LDS round trip per four entries).
+    auto each4 = [&](uint32_t* sl, auto&& f) {
+        for (int c0 = lane; c0 < seq_k; c0 += 256) {
+            uint32_t v[4];
+            #pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = sl[c0 + 64 * u < seq_k ? c0 + 64 * u : c0];
+            #pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = f(v[u]);
+            #pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (c0 + 64 * u < seq_k) sl[c0 + 64 * u] = v[u];
+        }
+    };
+    #pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        if (j ? has1 : has0) {
+            uint32_t* sl = slot + (j ? q1i : q0i) * seq_cap;
+            float m = -3.402823466e+38f;
+            for (int c0 = lane; c0 < seq_k; c0 += 256) {
+                uint32_t v[4];
+                #pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = sl[c0 + 64 * u < seq_k ? c0 + 64 * u : c0];
+                #pragma unroll
+                for (int u = 0; u < 4; ++u) m = fmaxf(m, h_f(static_cast<uint16_t>(v[u])));
+            }
+            for (int s = 32; s > 0; s >>= 1) m = fmaxf(m, __shfl_xor(m, s, 64));
+            each4(sl, [m](uint32_t v) { return __float_as_uint(exp_poly(h_f(static_cast<uint16_t>(v)) - m)); });
+        }
+    }
+    __syncthreads();
+    // denominators: lanes 0 and 1 of a wavefront, one query each, keys in index order (sixteen
+    // entries are read ahead of their additions; rows of slot start at multiples of 16 bytes)
+    {
+        const int qi = w + 4 * lane;
+        if (lane < 2 && qi < nrep) {
+            const uint32_t* sl = slot + qi * seq_cap;
+            float sum = 0.0f;
+            int c = 0;
+            for (; c + 16 <= seq_k; c += 16) {
+                uint4 v[4];
+                #pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const uint4*>(sl + c + 4 * u);
+                #pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    sum = sum + __uint_as_float(v[u].x);
+                    sum = sum + __uint_as_float(v[u].y);
+                    sum = sum + __uint_as_float(v[u].z);
+                    sum = sum + __uint_as_float(v[u].w);
+                }
+            }
+            for (; c < seq_k; ++c) sum = sum + __uint_as_float(sl[c]);
+            inv_s[qi] = rcp_rn(sum + 1e-20f);
+        }
+    }
+    __syncthreads();
+    // probabilities: fp16(fp16(e) * inv), as the separate kernels store them
+    #pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        if (j ? has1 : has0) {
+            const int qi = j ? q1i : q0i;
+            const float inv = inv_s[qi];
+            each4(slot + qi * seq_cap, [inv](uint32_t v) -> uint32_t { return f_h(h_f(f_h(__uint_as_float(v))) * inv); });
+        }
+    }
+    // values: thread (e = tid % D, tid / D) owns element e of queries tid / D + j (256 / D)
+    constexpr int kStep = 256 / D, kJ = 8 / kStep;
+    const int e = tid % D, qfirst = tid / D;
+    int qc[kJ];
+    float acc[kJ];
+    #pragma unroll
+    for (int j = 0; j < kJ; ++j) {
+        const int qi = qfirst + j * kStep;
+        qc[j] = (qi < nrep ? qi : nrep - 1) * seq_cap;
+        acc[j] = 0.0f;
+    }
+    for (int t0 = 0; t0 < seq_k; t0 += TK) {
+        const int rows = seq_k - t0 < TK ? seq_k - t0 : TK;
+        __syncthreads();                                             // probabilities are in place; the last tile has been used
+        stash(D);
+        __syncthreads();
+        if (t0 + TK < seq_k) fetch(vc, t0 + TK);
+        int r = 0;
+        for (; r + 8 <= rows; r += 8) {                              // eight keys read ahead of their sums
+            uint16_t v[8];
+            uint4 pr[kJ][2];
+            #pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = tile[(r + u) * D + e];
+            #pragma unroll
+            for (int j = 0; j < kJ; ++j) {
+                pr[j][0] = *reinterpret_cast<const uint4*>(slot + qc[j] + t0 + r);
+                pr[j][1] = *reinterpret_cast<const uint4*>(slot + qc[j] + t0 + r + 4);
+            }
+            #pragma unroll
+            for (int j = 0; j < kJ; ++j) {
+                const uint32_t p8[8] = {pr[j][0].x, pr[j][0].y, pr[j][0].z, pr[j][0].w, pr[j][1].x, pr[j][1].y, pr[j][1].z, pr[j][1].w};
+                #pragma unroll
+                for (int u = 0; u < 8; ++u) acc[j] = fmaf(h_f(static_cast<uint16_t>(p8[u])), h_f(v[u]), acc[j]);
+            }
+        }
+        for (; r < rows; ++r) {
+            const float v = h_f(tile[r * D + e]);
+            #pragma unroll
+            for (int j = 0; j < kJ; ++j) acc[j] = fmaf(h_f(static_cast<uint16_t>(slot[qc[j] + t0 + r])), v, acc[j]);
+        }
+    }
+    #pragma unroll
+    for (int j = 0; j < kJ; ++j) {
+        const int qi = qfirst + j * kStep;
+        if (qi < nrep) out[static_cast<size_t>(row) * qd + (static_cast<size_t>(g) * nrep + qi) * D + e] = f_h(acc[j]);
+    }
+}
+
+inline size_t group_attention_lds(int D, int nrep, int seq_cap) {
+    return static_cast<size_t>(16) * D + 2 * static_cast<size_t>(kPromptTile) * (D + 4) + 4 * static_cast<size_t>(nrep) * seq_cap;
 }
 
 // H[i] = fp16(H[i] + T[i]): the element-wise add behind a projection (QW/kernels/utils.cl element_add)
@@ -957,14 +1165,26 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
     const long nH = static_cast<long>(M) * Hd, nI = static_cast<long>(M) * I;
     const unsigned gH = static_cast<unsigned>(nH / 256 + 1 < 4096 ? nH / 256 + 1 : 4096);
     const unsigned gI = static_cast<unsigned>(nI / 256 + 1 < 8192 ? nI / 256 + 1 : 8192);
-    const size_t att_lds = static_cast<size_t>(D) * 2 + static_cast<size_t>(pos0 + M) * 6;
+    const size_t att_lds = static_cast<size_t>(D) * 2 * (1 + kPromptTile) + static_cast<size_t>(pos0 + M) * 6;
     if (att_lds > 65536) {
         static bool raised = false;
         if (!raised && !MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_rows_kernel),
                                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                      D * 2 + kMaxPositions * 6)))
+                                                      D * 2 * (1 + kPromptTile) + kMaxPositions * 6)))
             return 0;
         raised = true;
+    }
+    // one block per key/value head and row where the group's scores fit the LDS of a CU (160 KB, less
+    // the kernel's few static bytes)
+    constexpr size_t kGroupLdsMost = 160 * 1024 - 256;
+    const int nrep = c.n_heads / c.n_kv_heads;
+    const int grp_cap = (pos0 + M + 3) & ~3;             // rows of (query, key) entries start at multiples of 16 bytes
+    const size_t grp_lds = group_attention_lds(D, nrep, grp_cap);
+    const bool grouped = (D == 64 || D == 128) && nrep <= 8 && grp_lds <= kGroupLdsMost;
+    if (grouped && grp_lds > 65536) {
+        const void* kern = D == 64 ? reinterpret_cast<const void*>(attention_group_kernel<64>)
+                                   : reinterpret_cast<const void*>(attention_group_kernel<128>);
+        if (!MI_HIP_OK(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kGroupLdsMost)))) return 0;
     }
     for (int l = 0; l < c.n_layers; ++l) {
         hipLaunchKernelGGL(rmsnorm_kernel, dim3(M), dim3(64), 0, s, H, static_cast<const uint16_t*>(d->in_norm[l]), XN, Hd,
@@ -979,8 +1199,15 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
                            static_cast<const uint16_t*>(d->bk[l]), static_cast<const uint16_t*>(d->bv[l]), d->cosT, d->sinT,
                            kc, vc, QR, pos0, c.n_heads, c.n_kv_heads, D);
         if (!launched()) return 0;
-        hipLaunchKernelGGL(attention_rows_kernel, dim3(c.n_heads, M), dim3(256), att_lds, s, QR, kc, vc, ATT, pos0, pos0 + M,
-                           c.n_heads, c.n_kv_heads, D, scale);
+        if (grouped && D == 64)
+            hipLaunchKernelGGL(attention_group_kernel<64>, dim3(c.n_kv_heads, M), dim3(256), grp_lds, s, QR, kc, vc, ATT, pos0,
+                               grp_cap, c.n_heads, c.n_kv_heads, scale);
+        else if (grouped)
+            hipLaunchKernelGGL(attention_group_kernel<128>, dim3(c.n_kv_heads, M), dim3(256), grp_lds, s, QR, kc, vc, ATT, pos0,
+                               grp_cap, c.n_heads, c.n_kv_heads, scale);
+        else
+            hipLaunchKernelGGL(attention_rows_kernel, dim3(c.n_heads, M), dim3(256), att_lds, s, QR, kc, vc, ATT, pos0, pos0 + M,
+                               c.n_heads, c.n_kv_heads, D, scale);
         if (!launched()) return 0;
         if (!mi_linear(stream, M, Hd, qd, ATT, d->wo[l], T)) return 0;
         hipLaunchKernelGGL(add_rows_kernel, dim3(gH), dim3(256), 0, s, H, T, nH);
