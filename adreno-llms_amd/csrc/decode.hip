@@ -587,7 +587,7 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(const uint16_t* __r
 // pair owns 4 bytes of LDS that hold, in turn, its fp16 score, its fp32 exponential and its fp16
 // probability.  Wavefront w serves queries w and w + 4 in every phase but the last, where a thread
 // owns one output element of up to 8 D / 256 queries.
-// Dynamic LDS: 16 D + 2 kPromptTile (D + 4) + 4 nrep seq_cap bytes; seq_cap is a multiple of 4.
+// Dynamic LDS: 2 kPromptTile (D + 4) + 4 nrep seq_cap bytes; seq_cap is a multiple of 4.
 template <int D>
 __global__ __launch_bounds__(256) void attention_group_kernel(const uint16_t* __restrict__ QR, const uint16_t* __restrict__ kc,
                                                               const uint16_t* __restrict__ vc, uint16_t* __restrict__ out,
@@ -595,17 +595,22 @@ __global__ __launch_bounds__(256) void attention_group_kernel(const uint16_t* __
     typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
     constexpr int TK = kPromptTile, KS = D + 4, D4 = D / 4;
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-    uint16_t* qv = smem;                                            // [8][D]
-    uint16_t* tile = qv + 8 * D;                                    // [TK][KS] keys, then [TK][D] values
+    uint16_t* tile = smem;                                          // [TK][KS] keys, then [TK][D] values
     uint32_t* slot = reinterpret_cast<uint32_t*>(tile + TK * KS);   // [nrep][seq_cap]
     __shared__ float inv_s[8];
     const int g = blockIdx.x, row = blockIdx.y, pos = pos0 + row, seq_k = pos + 1;
     const int nrep = n_heads / n_kv_heads, kvd = n_kv_heads * D, qd = n_heads * D;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const uint16_t* qsrc = QR + static_cast<size_t>(row) * qd + static_cast<size_t>(g) * nrep * D;   // the group's heads are adjacent
-    for (int i = tid; i < nrep * D; i += 256) qv[i] = qsrc[i];
     const bool has0 = w < nrep, has1 = w + 4 < nrep;
     const int q0i = has0 ? w : 0, q1i = has1 ? w + 4 : q0i;
+    // the wavefront's two query rows live in registers for the whole scores phase
+    u16x4 qa[D4], qb[D4];
+    #pragma unroll
+    for (int d4 = 0; d4 < D4; ++d4) {
+        qa[d4] = *reinterpret_cast<const u16x4*>(qsrc + q0i * D + 4 * d4);
+        qb[d4] = *reinterpret_cast<const u16x4*>(qsrc + q1i * D + 4 * d4);
+    }
 
     // A tile's rows travel global memory -> registers -> LDS; the next tile's are requested before
     // the current tile is worked on, so that their latency runs under the arithmetic.
@@ -631,16 +636,14 @@ __global__ __launch_bounds__(256) void attention_group_kernel(const uint16_t* __
     fetch(kc, 0);
     for (int t0 = 0; t0 < seq_k; t0 += TK) {
         const int rows = seq_k - t0 < TK ? seq_k - t0 : TK;
-        __syncthreads();                                             // q is in place; the last tile has been used
+        __syncthreads();                                             // the last tile has been used
         stash(KS);
         __syncthreads();
         if (t0 + TK < seq_k) fetch(kc, t0 + TK);
         if (lane < rows) {
             const u16x4* kr = reinterpret_cast<const u16x4*>(tile + lane * KS);
-            const u16x4* qa = reinterpret_cast<const u16x4*>(qv + q0i * D);
-            const u16x4* qb = reinterpret_cast<const u16x4*>(qv + q1i * D);
             float acc0 = 0.0f, acc1 = 0.0f;
-            #pragma unroll 8
+            #pragma unroll
             for (int d4 = 0; d4 < D4; ++d4) {
                 const u16x4 b = kr[d4], a0 = qa[d4], a1 = qb[d4];
                 float t = h_f(a0[0]) * h_f(b[0]);
@@ -774,7 +777,7 @@ __global__ __launch_bounds__(256) void attention_group_kernel(const uint16_t* __
 }
 
 inline size_t group_attention_lds(int D, int nrep, int seq_cap) {
-    return static_cast<size_t>(16) * D + 2 * static_cast<size_t>(kPromptTile) * (D + 4) + 4 * static_cast<size_t>(nrep) * seq_cap;
+    return 2 * static_cast<size_t>(kPromptTile) * (D + 4) + 4 * static_cast<size_t>(nrep) * seq_cap;
 }
 
 // H[i] = fp16(H[i] + T[i]): the element-wise add behind a projection (QW/kernels/utils.cl element_add)
