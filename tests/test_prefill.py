@@ -161,3 +161,37 @@ def test_qwen_shaped_prompt_against_single_token_steps_on_device():
     finally:
         mil.lib().mi_set_gemm_mode(0)
         gd.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,cfg,n_prompt", [
+    # head_dim 128, four query heads per key/value head, three tiles of 64 cache rows, the cache filled to its last row
+    ("wide_heads", dict(hidden=1024, inter=1536, n_heads=8, n_kv_heads=2, head_dim=128, n_layers=2, vocab=2048,
+                        max_pos=150, rms_eps=1e-6, rope_theta=500000.0), 141),
+    # nine query heads per key/value head: more than a block of the grouped kernel serves, one block per head and row
+    ("nine_per_group", dict(hidden=576, inter=1536, n_heads=9, n_kv_heads=1, head_dim=64, n_layers=1, vocab=1024,
+                            max_pos=80, rms_eps=1e-5, rope_theta=100000.0), 71),
+    # eight heads per group over 1800 positions: 66 KB of scores per block, beyond the 64 KB a kernel gets
+    # unasked; checked against the device's own single-token steps (the CPU harness would need 15 s)
+    ("long_context", dict(hidden=512, inter=512, n_heads=8, n_kv_heads=1, head_dim=64, n_layers=1, vocab=512,
+                          max_pos=1800, rms_eps=1e-6, rope_theta=1000000.0), 1800),
+])
+def test_prompt_other_geometries_bit_for_bit(name, cfg, n_prompt):
+    assert mil.lib().mi_init(0) == 1
+    mil.lib().mi_set_gemm_mode(1)
+    try:
+        queue = mil.Queue()
+        m = Model(cfg, seed=17)
+        prompt = _prompt(n_prompt, cfg["vocab"], 8)
+        gd = GpuDecoder(m, queue)
+        if name == "long_context":
+            want = gd.greedy(prompt, 1)
+            logits = gd.logits()
+        else:
+            want, _, logits = _oracle(m, prompt, 1)
+        assert gd.dec.prefill(queue, prompt)
+        assert gd.dec.read(queue) == (n_prompt, want[0])
+        assert np.array_equal(gd.logits(), logits)
+        gd.close()
+    finally:
+        mil.lib().mi_set_gemm_mode(0)
