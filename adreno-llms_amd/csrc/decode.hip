@@ -786,6 +786,63 @@ __global__ void add_rows_kernel(uint16_t* __restrict__ H, const uint16_t* __rest
         H[i] = f_h(h_f(T[i]) + h_f(H[i]));
 }
 
+// add_rows_kernel and rmsnorm_kernel in one launch, a wavefront per row: H[r] = fp16(H[r] + T[r]),
+// out[r] = rmsnorm(H[r]) * w, with the operations of the two kernels in their order (the row stays
+// in registers between them).  For rows of at most 2048 elements, a multiple of 4.
+__global__ __launch_bounds__(64) void add_rmsnorm_rows_kernel(uint16_t* __restrict__ H, const uint16_t* __restrict__ T,
+                                                              const uint16_t* __restrict__ w, uint16_t* __restrict__ out,
+                                                              int cols, float eps) {
+    constexpr int kGroups = 8;
+    typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+    const int lid = threadIdx.x, c4n = cols >> 2;
+    H += static_cast<size_t>(blockIdx.x) * cols;
+    T += static_cast<size_t>(blockIdx.x) * cols;
+    out += static_cast<size_t>(blockIdx.x) * cols;
+    u16x4 xv[kGroups], tv[kGroups], wv[kGroups];
+    #pragma unroll
+    for (int g = 0; g < kGroups; ++g) {
+        const int c4 = lid + 64 * g;
+        if (c4 < c4n) {
+            xv[g] = *reinterpret_cast<const u16x4*>(H + 4 * c4);
+            tv[g] = *reinterpret_cast<const u16x4*>(T + 4 * c4);
+            wv[g] = *reinterpret_cast<const u16x4*>(w + 4 * c4);
+        }
+    }
+    float acc = 0.0f;
+    #pragma unroll
+    for (int g = 0; g < kGroups; ++g) {
+        const int c4 = lid + 64 * g;
+        if (c4 < c4n) {
+            #pragma unroll
+            for (int e = 0; e < 4; ++e) xv[g][e] = f_h(h_f(tv[g][e]) + h_f(xv[g][e]));
+            *reinterpret_cast<u16x4*>(H + 4 * c4) = xv[g];
+            const float v0 = h_f(xv[g][0]), v1 = h_f(xv[g][1]), v2 = h_f(xv[g][2]), v3 = h_f(xv[g][3]);
+            float d = v0 * v0;
+            d = fmaf(v1, v1, d);
+            d = fmaf(v2, v2, d);
+            d = fmaf(v3, v3, d);
+            acc = acc + d;
+        }
+    }
+    #pragma unroll
+    for (int s = 32; s > 0; s >>= 1) {
+        const float o = __shfl_down(acc, s, 64);
+        acc = acc + o;
+    }
+    const float total = __shfl(acc, 0, 64);
+    const float inv = rcp_rn(sqrtf(__fdiv_rn(total, static_cast<float>(cols)) + eps));
+    #pragma unroll
+    for (int g = 0; g < kGroups; ++g) {
+        const int c4 = lid + 64 * g;
+        if (c4 < c4n) {
+            u16x4 o;
+            #pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = f_h((h_f(xv[g][e]) * inv) * h_f(wv[g][e]));
+            *reinterpret_cast<u16x4*>(out + 4 * c4) = o;
+        }
+    }
+}
+
 // gate[i] = swiglu(gate[i], up[i]) over any number of elements (swiglu_kernel takes an int count)
 __global__ void swiglu_rows_kernel(uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, long n) {
     for (long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += static_cast<long>(gridDim.x) * blockDim.x) {
@@ -1189,10 +1246,23 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
                                    : reinterpret_cast<const void*>(attention_group_kernel<128>);
         if (!MI_HIP_OK(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kGroupLdsMost)))) return 0;
     }
+    // H += T, then XN = rmsnorm(H) * w: one launch where a row fits the fused kernel's registers
+    const bool add_norm_fused = Hd % 4 == 0 && Hd <= 2048;
+    auto add_then_norm = [&](const void* w) {
+        if (add_norm_fused) {
+            hipLaunchKernelGGL(add_rmsnorm_rows_kernel, dim3(M), dim3(64), 0, s, H, T, static_cast<const uint16_t*>(w), XN, Hd,
+                               c.rms_eps);
+            return launched();
+        }
+        hipLaunchKernelGGL(add_rows_kernel, dim3(gH), dim3(256), 0, s, H, T, nH);
+        if (!launched()) return false;
+        hipLaunchKernelGGL(rmsnorm_kernel, dim3(M), dim3(64), 0, s, H, static_cast<const uint16_t*>(w), XN, Hd, c.rms_eps);
+        return launched();
+    };
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(M), dim3(64), 0, s, H, static_cast<const uint16_t*>(d->in_norm[0]), XN, Hd,
+                       c.rms_eps);
+    if (!launched()) return 0;
     for (int l = 0; l < c.n_layers; ++l) {
-        hipLaunchKernelGGL(rmsnorm_kernel, dim3(M), dim3(64), 0, s, H, static_cast<const uint16_t*>(d->in_norm[l]), XN, Hd,
-                           c.rms_eps);
-        if (!launched()) return 0;
         if (!mi_linear(stream, M, qd, Hd, XN, d->wq[l], Q) || !mi_linear(stream, M, kvd, Hd, XN, d->wk[l], Kp) ||
             !mi_linear(stream, M, kvd, Hd, XN, d->wv[l], V))
             return 0;
@@ -1213,17 +1283,17 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
                                c.n_heads, c.n_kv_heads, D, scale);
         if (!launched()) return 0;
         if (!mi_linear(stream, M, Hd, qd, ATT, d->wo[l], T)) return 0;
-        hipLaunchKernelGGL(add_rows_kernel, dim3(gH), dim3(256), 0, s, H, T, nH);
-        if (!launched()) return 0;
-        hipLaunchKernelGGL(rmsnorm_kernel, dim3(M), dim3(64), 0, s, H, static_cast<const uint16_t*>(d->post_norm[l]), XN, Hd,
-                           c.rms_eps);
-        if (!launched()) return 0;
+        if (!add_then_norm(d->post_norm[l])) return 0;
         if (!mi_linear(stream, M, I, Hd, XN, d->wgate[l], G) || !mi_linear(stream, M, I, Hd, XN, d->wup[l], U)) return 0;
         hipLaunchKernelGGL(swiglu_rows_kernel, dim3(gI), dim3(256), 0, s, G, U, nI);
         if (!launched()) return 0;
         if (!mi_linear(stream, M, Hd, I, G, d->wdown[l], T)) return 0;
-        hipLaunchKernelGGL(add_rows_kernel, dim3(gH), dim3(256), 0, s, H, T, nH);
-        if (!launched()) return 0;
+        if (l + 1 < c.n_layers) {
+            if (!add_then_norm(d->in_norm[l + 1])) return 0;     // the next layer's input norm rides along
+        } else {
+            hipLaunchKernelGGL(add_rows_kernel, dim3(gH), dim3(256), 0, s, H, T, nH);
+            if (!launched()) return 0;
+        }
     }
     // only the last position picks a token: its residual stream becomes the single-token state
     if (!MI_HIP_OK(hipMemcpyAsync(d->h, H + static_cast<size_t>(M - 1) * Hd, static_cast<size_t>(Hd) * 2,
