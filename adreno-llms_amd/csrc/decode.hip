@@ -843,12 +843,21 @@ __global__ __launch_bounds__(64) void add_rmsnorm_rows_kernel(uint16_t* __restri
     }
 }
 
-// gate[i] = swiglu(gate[i], up[i]) over any number of elements (swiglu_kernel takes an int count)
+// gate[i] = swiglu(gate[i], up[i]) over any number of elements, four per thread and step (n is a
+// multiple of 4 and both arrays start at multiples of 8 bytes; swiglu_kernel's operations per element)
 __global__ void swiglu_rows_kernel(uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, long n) {
-    for (long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += static_cast<long>(gridDim.x) * blockDim.x) {
-        const float g = h_f(gate[i]), u = h_f(up[i]);
-        const float sig = rcp_rn(1.0f + exp_poly(-g));
-        gate[i] = f_h((g * sig) * u);
+    typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+    const long n4 = n >> 2;
+    for (long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += static_cast<long>(gridDim.x) * blockDim.x) {
+        u16x4 g4 = *reinterpret_cast<const u16x4*>(gate + 4 * i);
+        const u16x4 u4 = *reinterpret_cast<const u16x4*>(up + 4 * i);
+        #pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float g = h_f(g4[e]), u = h_f(u4[e]);
+            const float sig = rcp_rn(1.0f + exp_poly(-g));
+            g4[e] = f_h((g * sig) * u);
+        }
+        *reinterpret_cast<u16x4*>(gate + 4 * i) = g4;
     }
 }
 
@@ -1224,7 +1233,7 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
     if (!launched()) return 0;
     const long nH = static_cast<long>(M) * Hd, nI = static_cast<long>(M) * I;
     const unsigned gH = static_cast<unsigned>(nH / 256 + 1 < 4096 ? nH / 256 + 1 : 4096);
-    const unsigned gI = static_cast<unsigned>(nI / 256 + 1 < 8192 ? nI / 256 + 1 : 8192);
+    const unsigned gI = static_cast<unsigned>(nI / 1024 + 1 < 8192 ? nI / 1024 + 1 : 8192);
     const size_t att_lds = static_cast<size_t>(D) * 2 * (1 + kPromptTile) + static_cast<size_t>(pos0 + M) * 6;
     if (att_lds > 65536) {
         static bool raised = false;
@@ -1285,7 +1294,12 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
         if (!mi_linear(stream, M, Hd, qd, ATT, d->wo[l], T)) return 0;
         if (!add_then_norm(d->post_norm[l])) return 0;
         if (!mi_linear(stream, M, I, Hd, XN, d->wgate[l], G) || !mi_linear(stream, M, I, Hd, XN, d->wup[l], U)) return 0;
-        hipLaunchKernelGGL(swiglu_rows_kernel, dim3(gI), dim3(256), 0, s, G, U, nI);
+        if (I % 4 == 0) {
+            hipLaunchKernelGGL(swiglu_rows_kernel, dim3(gI), dim3(256), 0, s, G, U, nI);
+        } else {
+            if (nI > 2147483647L) return 0;
+            hipLaunchKernelGGL(swiglu_kernel, dim3(gI), dim3(256), 0, s, G, U, static_cast<int>(nI));
+        }
         if (!launched()) return 0;
         if (!mi_linear(stream, M, Hd, I, G, d->wdown[l], T)) return 0;
         if (l + 1 < c.n_layers) {

@@ -95,7 +95,8 @@ def test_prompt_in_two_parts_and_after_steps():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name,cfg,n_prompt", [("smol", SMOL, 40), ("tiny", TINY, 33)])
+@pytest.mark.parametrize("name,cfg,n_prompt", [("smol", SMOL, 40), ("tiny", TINY, 33), ("smol-f16", SMOL, 40),
+                                               ("smol-q4", SMOL, 40)])
 def test_prompt_on_the_matrix_cores_within_tolerance(name, cfg, n_prompt):
     """Default mode: the M-row projections run as MFMA GEMMs where the library's estimate favours
     them.  Each projection is within one fp16 step of the rows of GEMV; through the layers of the
@@ -104,9 +105,10 @@ def test_prompt_on_the_matrix_cores_within_tolerance(name, cfg, n_prompt):
     margin exceeds twice the largest difference."""
     assert mil.lib().mi_init(0) == 1
     queue = mil.Queue()
-    m = Model(cfg, seed=33)
+    kind = name.split("-")[1] if "-" in name else "i8"
+    m = Model(cfg, seed=33) if kind == "i8" else KindModel(cfg, kind, seed=33)
     prompt = _prompt(n_prompt, cfg["vocab"], 5)
-    want, margins, logits = _oracle(m, prompt, 1)
+    want, margins, logits = _oracle(m, prompt, 1, linear_cb=None if kind == "i8" else m.oracle_cb())
     gd = GpuDecoder(m, queue)
     assert gd.dec.prefill(queue, prompt)
     pos, tok = gd.dec.read(queue)
