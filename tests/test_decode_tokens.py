@@ -115,11 +115,24 @@ def test_qwen_shaped_whole_step_on_device_graph_replay():
     got = gd.greedy(PROMPT, 32, graph=True)
     got_logits = gd.logits()
     pos, _ = gd.dec.read(queue)
+    # the same 32 tokens with the prompt taken at once (projections as rows of GEMV: bit-identical)
+    mil.lib().mi_set_gemm_mode(1)
+    try:
+        assert gd.dec.prefill(queue, PROMPT)
+        again = [gd.dec.read(queue)[1]]
+        for _ in range(31):
+            assert gd.dec.step(queue)
+            again.append(gd.dec.read(queue)[1])
+        again_logits = gd.logits()
+    finally:
+        mil.lib().mi_set_gemm_mode(0)
     gd.close()
     print("tokens", got, flush=True)
     assert got == want
     assert np.array_equal(got_logits, want_logits)      # every bit of the last step's 151936 logits
     assert pos == len(PROMPT) - 1 + 32       # the first prompt token is set by reset, every later token costs a step
+    assert again == want
+    assert np.array_equal(again_logits, want_logits)
 
 
 @pytest.mark.gpu
