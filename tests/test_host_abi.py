@@ -70,6 +70,8 @@ int main(void) {
     mi_decoder_config cfg;
     memset(&cfg, 0, sizeof cfg);
     if (mi_decoder_create(&cfg, 0) != 0) return 3;          /* refused: bad configuration, no device touched */
+    int tok = 0;
+    if (mi_decoder_prefill(0, 0, &tok, 1, 0) != 0) return 4;    /* refused: no decoder, no device touched */
     printf("ok %d %d\n", (int)q[0], (int)p[0]);
     return 0;
 }
