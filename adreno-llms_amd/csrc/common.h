@@ -90,6 +90,8 @@ bool fused_gemv(hipStream_t s, int n, const int* N, int K, const void* x, const 
 bool linear_argmax(hipStream_t s, int N, int K, const void* x, const void* W, void* logits, const void* norm_w,
                    float norm_eps, int num_partials, void* token_out, int* token_copy, int* counter, bool* taken);
 bool fused_gemv_kind(const void* W, int N, int K, WeightKind* kind);   // kind W is registered as (fp16 if not)
+// The same with the scales W was registered with (null for fp16 weights).
+bool registered_weight(const void* W, int N, int K, WeightKind* kind, const void** scale);
 
 // argmax.hip: index of the greatest of N fp16 values, ties as the reference's two argmax kernels break them.
 // scratch: kArgmaxScratchBytes of device memory that belongs to stream s, or null (then one block does all the work).

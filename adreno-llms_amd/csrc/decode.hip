@@ -475,7 +475,10 @@ __global__ __launch_bounds__(256) void rope_rows_kernel(const uint16_t* __restri
                                                         const uint16_t* __restrict__ bk, const uint16_t* __restrict__ bv,
                                                         const uint16_t* __restrict__ cosT, const uint16_t* __restrict__ sinT,
                                                         uint16_t* __restrict__ kc, uint16_t* __restrict__ vc,
-                                                        uint16_t* __restrict__ QR, int pos0, int n_heads, int n_kv_heads, int D) {
+                                                        uint16_t* __restrict__ QR, int pos0, int n_heads, int n_kv_heads, int D,
+                                                        int ldq, int ldkv) {
+    // ldq, ldkv: halves between rows of Q and of Kp / V (the widths of the projections, or of the
+    // stacked q|k|v projection they are columns of)
     const int row = blockIdx.x, pos = pos0 + row, hd2 = D / 2, qd = n_heads * D, kvd = n_kv_heads * D;
     const uint16_t* cr = cosT + static_cast<size_t>(pos) * D;
     const uint16_t* sr = sinT + static_cast<size_t>(pos) * D;
@@ -483,7 +486,7 @@ __global__ __launch_bounds__(256) void rope_rows_kernel(const uint16_t* __restri
         const int head = j / hd2, i = j - head * hd2;
         const bool isq = head < n_heads;
         const int hh = isq ? head : head - n_heads;
-        const uint16_t* buf = isq ? Q + static_cast<size_t>(row) * qd + hh * D : Kp + static_cast<size_t>(row) * kvd + hh * D;
+        const uint16_t* buf = isq ? Q + static_cast<size_t>(row) * ldq + hh * D : Kp + static_cast<size_t>(row) * ldkv + hh * D;
         const uint16_t* bias = (isq ? bq : bk) + hh * D;
         uint16_t* dst = isq ? QR + static_cast<size_t>(row) * qd + hh * D : kc + static_cast<size_t>(pos) * kvd + hh * D;
         const float c = h_f(cr[i]), sn = h_f(sr[i]);
@@ -493,7 +496,7 @@ __global__ __launch_bounds__(256) void rope_rows_kernel(const uint16_t* __restri
         dst[i + hd2] = f_h(fmaf(x2, c, x1 * sn));
     }
     for (int e = threadIdx.x; e < kvd; e += blockDim.x)
-        vc[static_cast<size_t>(pos) * kvd + e] = f_h(h_f(V[static_cast<size_t>(row) * kvd + e]) + h_f(bv[e]));
+        vc[static_cast<size_t>(pos) * kvd + e] = f_h(h_f(V[static_cast<size_t>(row) * ldkv + e]) + h_f(bv[e]));
 }
 
 // One block per (query head, row): the query of position pos0 + row against cache rows
@@ -861,6 +864,26 @@ __global__ void swiglu_rows_kernel(uint16_t* __restrict__ gate, const uint16_t* 
     }
 }
 
+// out[r][c] = swiglu(GU[r][c], GU[r][inter + c]): rows of a stacked gate|up projection ([M, 2 inter]),
+// four columns per thread and step (inter a multiple of 4); swiglu_kernel's operations per element
+__global__ void swiglu_stacked_kernel(const uint16_t* __restrict__ GU, uint16_t* __restrict__ out, int inter, long n4) {
+    typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+    const int c4n = inter >> 2;
+    for (long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += static_cast<long>(gridDim.x) * blockDim.x) {
+        const long r = i / c4n;
+        const int c = static_cast<int>(i - r * c4n) * 4;
+        u16x4 g4 = *reinterpret_cast<const u16x4*>(GU + r * 2 * inter + c);
+        const u16x4 u4 = *reinterpret_cast<const u16x4*>(GU + r * 2 * inter + inter + c);
+        #pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float g = h_f(g4[e]), u = h_f(u4[e]);
+            const float sig = rcp_rn(1.0f + exp_poly(-g));
+            g4[e] = f_h((g * sig) * u);
+        }
+        *reinterpret_cast<u16x4*>(out + r * inter + c) = g4;
+    }
+}
+
 // the state a prompt leaves behind for the launches that pick the next token: they read the
 // last prompt position and advance it
 __global__ void set_pos_kernel(State* st, int pos) { st->pos = pos; }
@@ -894,6 +917,11 @@ struct Decoder {
     // only for a longer one
     void* prompt_mem = nullptr;
     int prompt_rows = 0;
+    // q|k|v and gate|up of every layer as one matrix each (rows stacked, scales stacked), copies made
+    // with the first prompt: a prompt's projections of one input are then one GEMM instead of three
+    // or two.  An entry stays null where a layer's matrices are not of one kind.
+    std::vector<void*> wqkv, wgu, stacked_mem;
+    bool stacked_built = false;
 };
 
 template <typename T>
@@ -994,6 +1022,9 @@ int mi_decoder_destroy(void* dec) {
     if (!d) return 1;
     for (void* p : d->owned) (void)hipFree(p);
     if (d->prompt_mem) (void)hipFree(d->prompt_mem);
+    for (void* w : d->wqkv) if (w) mi_unregister_weight(w);
+    for (void* w : d->wgu) if (w) mi_unregister_weight(w);
+    for (void* p : d->stacked_mem) (void)hipFree(p);
     delete d;
     return 1;
 }
@@ -1185,6 +1216,39 @@ int mi_decoder_step(void* dec, void* stream) {
     return decoder_pick_next(d, stream);
 }
 
+// Rows of n matrices of one kind and K (and their scales) copied into one matrix, registered like
+// its parts.  Null when the parts are not of one kind or memory is short; *failed on a HIP error.
+static void* stack_weights(Decoder* d, hipStream_t s, int n, const void* const* W, const int* N, int K, bool* failed) {
+    WeightKind kind = WK_F16, k0 = WK_F16;
+    const void* scale[4] = {nullptr, nullptr, nullptr, nullptr};
+    int total = 0;
+    for (int i = 0; i < n; ++i) {
+        if (!registered_weight(W[i], N[i], K, &kind, &scale[i])) return nullptr;
+        if (i == 0) k0 = kind;
+        if (kind != k0) return nullptr;
+        total += N[i];
+    }
+    const size_t row = k0 == WK_F16 ? static_cast<size_t>(K) * 2 : k0 == WK_I8 ? static_cast<size_t>(K) : static_cast<size_t>(K) / 2;
+    const size_t srow = k0 == WK_I8 ? 2 : k0 == WK_Q4 ? static_cast<size_t>(K / 32) * 2 : 0;
+    void *w = nullptr, *sc = nullptr;
+    if (hipMalloc(&w, row * total) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    d->stacked_mem.push_back(w);
+    if (srow) {
+        if (hipMalloc(&sc, srow * total) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+        d->stacked_mem.push_back(sc);
+    }
+    size_t at = 0;
+    for (int i = 0; i < n; ++i) {
+        bool ok = MI_HIP_OK(hipMemcpyAsync(static_cast<char*>(w) + at * row, W[i], row * N[i], hipMemcpyDeviceToDevice, s));
+        if (ok && srow)
+            ok = MI_HIP_OK(hipMemcpyAsync(static_cast<char*>(sc) + at * srow, scale[i], srow * N[i], hipMemcpyDeviceToDevice, s));
+        if (!ok) { *failed = true; return nullptr; }
+        at += N[i];
+    }
+    const int reg = k0 == WK_I8 ? mi_register_int8_weight(w, sc, total, K) : k0 == WK_Q4 ? mi_register_q4_weight(w, sc, total, K) : 1;
+    return reg ? w : nullptr;
+}
+
 int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens, int pos0) {
     auto* d = static_cast<Decoder*>(dec);
     if (!d || !tokens || n_tokens < 1 || pos0 < 0 || static_cast<long>(pos0) + n_tokens > d->c.max_pos) {
@@ -1198,9 +1262,11 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
     const float scale = 1.0f / sqrtf(static_cast<float>(D));
     auto launched = [] { return MI_HIP_OK(hipGetLastError()); };
 
-    // rows of the prompt: H, XN, T [M, hidden]; Q, QR, ATT [M, qd]; K, V [M, kvd]; G, U [M, inter]; tokens
+    // rows of the prompt: H, XN, T [M, hidden]; QKV [M, qd + 2 kvd] (q | k | v of a row side by side
+    // from the stacked projection, or three blocks of their own); QR, ATT [M, qd]; GU [M, 2 inter]
+    // likewise; G2 [M, inter]; tokens
     const size_t row_halves = 3 * static_cast<size_t>(Hd) + 3 * static_cast<size_t>(qd) + 2 * static_cast<size_t>(kvd) +
-                              2 * static_cast<size_t>(I);
+                              3 * static_cast<size_t>(I);
     if (M > d->prompt_rows) {
         if (d->prompt_mem) {
             if (!MI_HIP_OK(hipStreamSynchronize(s))) return 0;      // an earlier prompt may still be running in it
@@ -1224,10 +1290,25 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
         at += (halves_per_row * cap + 7) & ~static_cast<size_t>(7);
         return p;
     };
-    uint16_t *H = carve(Hd), *XN = carve(Hd), *T = carve(Hd), *Q = carve(qd), *QR = carve(qd), *ATT = carve(qd);
-    uint16_t *Kp = carve(kvd), *V = carve(kvd), *G = carve(I), *U = carve(I);
+    uint16_t *H = carve(Hd), *XN = carve(Hd), *T = carve(Hd), *QKV = carve(qd + 2 * kvd), *QR = carve(qd), *ATT = carve(qd);
+    uint16_t *GU = carve(2 * static_cast<size_t>(I)), *G2 = carve(I);
     int* tok = reinterpret_cast<int*>(base + at);
 
+    if (!d->stacked_built) {
+        d->wqkv.assign(c.n_layers, nullptr);
+        d->wgu.assign(c.n_layers, nullptr);
+        bool failed = false;
+        for (int l = 0; l < c.n_layers && !failed; ++l) {
+            const void* const W3[3] = {d->wq[l], d->wk[l], d->wv[l]};
+            const int N3[3] = {qd, kvd, kvd};
+            d->wqkv[l] = stack_weights(d, s, 3, W3, N3, Hd, &failed);
+            const void* const W2[2] = {d->wgate[l], d->wup[l]};
+            const int N2[2] = {I, I};
+            if (!failed && I % 4 == 0) d->wgu[l] = stack_weights(d, s, 2, W2, N2, Hd, &failed);
+        }
+        if (failed) return 0;
+        d->stacked_built = true;
+    }
     if (!MI_HIP_OK(hipMemcpyAsync(tok, tokens, static_cast<size_t>(M) * 4, hipMemcpyHostToDevice, s))) return 0;
     hipLaunchKernelGGL(embed_rows_kernel, dim3(M), dim3(256), 0, s, static_cast<const uint16_t*>(d->embed), tok, H, Hd, c.vocab);
     if (!launched()) return 0;
@@ -1272,14 +1353,27 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
                        c.rms_eps);
     if (!launched()) return 0;
     for (int l = 0; l < c.n_layers; ++l) {
-        if (!mi_linear(stream, M, qd, Hd, XN, d->wq[l], Q) || !mi_linear(stream, M, kvd, Hd, XN, d->wk[l], Kp) ||
-            !mi_linear(stream, M, kvd, Hd, XN, d->wv[l], V))
-            return 0;
+        uint16_t *Q = QKV, *Kp, *V;
+        int ldq, ldkv;
+        if (d->wqkv[l]) {
+            if (!mi_linear(stream, M, qd + 2 * kvd, Hd, XN, d->wqkv[l], QKV)) return 0;
+            Kp = QKV + qd;
+            V = Kp + kvd;
+            ldq = ldkv = qd + 2 * kvd;
+        } else {
+            Kp = QKV + static_cast<size_t>(cap) * qd;
+            V = Kp + static_cast<size_t>(cap) * kvd;
+            ldq = qd;
+            ldkv = kvd;
+            if (!mi_linear(stream, M, qd, Hd, XN, d->wq[l], Q) || !mi_linear(stream, M, kvd, Hd, XN, d->wk[l], Kp) ||
+                !mi_linear(stream, M, kvd, Hd, XN, d->wv[l], V))
+                return 0;
+        }
         uint16_t* kc = d->kc + static_cast<size_t>(l) * c.max_pos * kvd;
         uint16_t* vc = d->vc + static_cast<size_t>(l) * c.max_pos * kvd;
         hipLaunchKernelGGL(rope_rows_kernel, dim3(M), dim3(256), 0, s, Q, Kp, V, static_cast<const uint16_t*>(d->bq[l]),
                            static_cast<const uint16_t*>(d->bk[l]), static_cast<const uint16_t*>(d->bv[l]), d->cosT, d->sinT,
-                           kc, vc, QR, pos0, c.n_heads, c.n_kv_heads, D);
+                           kc, vc, QR, pos0, c.n_heads, c.n_kv_heads, D, ldq, ldkv);
         if (!launched()) return 0;
         if (grouped && D == 64)
             hipLaunchKernelGGL(attention_group_kernel<64>, dim3(c.n_kv_heads, M), dim3(256), grp_lds, s, QR, kc, vc, ATT, pos0,
@@ -1293,15 +1387,24 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
         if (!launched()) return 0;
         if (!mi_linear(stream, M, Hd, qd, ATT, d->wo[l], T)) return 0;
         if (!add_then_norm(d->post_norm[l])) return 0;
-        if (!mi_linear(stream, M, I, Hd, XN, d->wgate[l], G) || !mi_linear(stream, M, I, Hd, XN, d->wup[l], U)) return 0;
-        if (I % 4 == 0) {
-            hipLaunchKernelGGL(swiglu_rows_kernel, dim3(gI), dim3(256), 0, s, G, U, nI);
+        const uint16_t* act;                      // swiglu(gate, up), [M, inter]
+        if (d->wgu[l]) {
+            if (!mi_linear(stream, M, 2 * I, Hd, XN, d->wgu[l], GU)) return 0;
+            hipLaunchKernelGGL(swiglu_stacked_kernel, dim3(gI), dim3(256), 0, s, GU, G2, I, nI / 4);
+            act = G2;
         } else {
-            if (nI > 2147483647L) return 0;
-            hipLaunchKernelGGL(swiglu_kernel, dim3(gI), dim3(256), 0, s, G, U, static_cast<int>(nI));
+            uint16_t *G = GU, *U = GU + static_cast<size_t>(cap) * I;
+            if (!mi_linear(stream, M, I, Hd, XN, d->wgate[l], G) || !mi_linear(stream, M, I, Hd, XN, d->wup[l], U)) return 0;
+            if (I % 4 == 0) {
+                hipLaunchKernelGGL(swiglu_rows_kernel, dim3(gI), dim3(256), 0, s, G, U, nI);
+            } else {
+                if (nI > 2147483647L) return 0;
+                hipLaunchKernelGGL(swiglu_kernel, dim3(gI), dim3(256), 0, s, G, U, static_cast<int>(nI));
+            }
+            act = G;
         }
         if (!launched()) return 0;
-        if (!mi_linear(stream, M, Hd, I, G, d->wdown[l], T)) return 0;
+        if (!mi_linear(stream, M, Hd, I, act, d->wdown[l], T)) return 0;
         if (l + 1 < c.n_layers) {
             if (!add_then_norm(d->in_norm[l + 1])) return 0;     // the next layer's input norm rides along
         } else {

@@ -82,6 +82,14 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
 const DeviceInfo& device_info() { return g_dev; }
 
+bool registered_weight(const void* W, int N, int K, WeightKind* kind, const void** scale) {
+    Entry e;
+    if (!resolve("decode step", W, N, K, &e)) return false;
+    *kind = e.kind;
+    *scale = e.scale;
+    return true;
+}
+
 bool fused_gemv_kind(const void* W, int N, int K, WeightKind* kind) {
     Entry e;
     if (!resolve("decode step", W, N, K, &e)) return false;

@@ -72,9 +72,12 @@ int   mi_decoder_step(void* decoder, void* stream);
  * calls of mi_decoder_step with the tokens forced would leave.  The cache rows and the logits
  * are those of such steps bit for bit when the M > 1 projections run as rows of GEMV
  * (mi_set_gemm_mode(1), the reference's quantised prefill, LF/src/model.cpp:243-250), and within
- * the GEMM's tolerance of them on the matrix cores.  pos0 + n_tokens <= max_pos.  The first prompt,
- * and any longer one later, allocates the prompt's activation rows (about 31 KB per token at
- * Qwen2.5-0.5B widths); not for graph capture.  mi_decoder_buffer(0) afterwards holds the residual
+ * the GEMM's tolerance of them on the matrix cores.  pos0 + n_tokens <= max_pos.  The first prompt
+ * makes device copies of every layer's q, k, v and gate, up matrices stacked into one matrix each
+ * (the reference's stacked qkv, QW/src/layers/attention.cpp:414; as much memory again as those
+ * matrices), so that the projections of one input are one GEMM; it, and any longer prompt later,
+ * allocates the prompt's activation rows (about 40 KB per token at Qwen2.5-0.5B widths).  Not for
+ * graph capture.  mi_decoder_buffer(0) afterwards holds the residual
  * stream of the last position; buffers 1 .. 5 are left as they were. */
 int   mi_decoder_prefill(void* decoder, void* stream, const int* tokens, int n_tokens, int pos0);
 
