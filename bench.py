@@ -275,18 +275,6 @@ def main():
             "launches_per_step": 24 * 5 + 3, "positions": f"8..{pos_after - 1}", "launch": "hip_graph"}
         dec.close()
 
-        # a prompt at once: the M-row projections of all 24 layers through the GEMM, the last
-        # position's lm_head and argmax; against M single-token steps at the rate measured above
-        big = mil.Decoder(dict(cfg, max_pos=2048), dec_w)
-        for M in (64, 512, 2048):
-            ids = [int(t) for t in np.random.default_rng(M).integers(0, VOCAB, M)]
-            assert big.prefill(queue, ids)
-            ms = time_region(mil, queue, lambda: big.prefill(queue, ids), 3)
-            detail[f"c5_whole_prompt_on_device_M{M}"] = {
-                "ms": round(ms, 3), "prompt_tokens_per_s": round(M / ms * 1e3, 0),
-                "vs_single_token_steps": round(M * ms_tok / ms, 1)}
-        big.close()
-
         # the same step with block-32 Q4 weights (the LFM2 bundles' format): norm and SwiGLU ride in the
         # exact Q4 GEMV, the lm_head takes the throughput kernel with the argmax in its epilogue
         q4_keep, q4_w = [], dict(dec_w)
@@ -384,6 +372,21 @@ def main():
                     "us": round(ms * 1e3, 2), "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 1),
                     "frac_mfma_fp16_peak": round(flop / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)}
         mil.nnopt_unregister_weight(wb)
+
+    # ---- a prompt at once (after the GEMM lines above, which it would otherwise disturb: it
+    # allocates and frees a few hundred MB) ----------------------------------------------
+    if not args.no_detail and not args.no_graph:
+        # a prompt at once: the M-row projections of all 24 layers through the GEMM, the last
+        # position's lm_head and argmax; against M single-token steps at the rate measured above
+        big = mil.Decoder(dict(cfg, max_pos=2048), dec_w)
+        for M in (64, 512, 2048):
+            ids = [int(t) for t in np.random.default_rng(M).integers(0, VOCAB, M)]
+            assert big.prefill(queue, ids)
+            ms = time_region(mil, queue, lambda: big.prefill(queue, ids), 3)
+            detail[f"c5_whole_prompt_on_device_M{M}"] = {
+                "ms": round(ms, 3), "prompt_tokens_per_s": round(M / ms * 1e3, 0),
+                "vs_single_token_steps": round(M * ms_tok / ms, 1)}
+        big.close()
 
     # ---- CPU baseline: the oracle on a bounded sample of the same sweep -------------------
     cpu = None
