@@ -18,9 +18,15 @@
  * Graph: QW/src/model.cpp:243-376, QW/src/layers/attention.cpp:336-674,
  * QW/src/layers/mlp.cpp:97-237.  The prompt is fed token by token through the same
  * step (the reference's quantised prefill is such a loop, LF/src/model.cpp:243-250).
- * These restatements are "parity unpinned" against the reference (no fixture of the
- * reference covers them without the real checkpoints); they only have to be the same
- * code on both sides of the comparison.
+ * Pins (tests/test_oracle_decode.py, CPU only): every function below against an fp64 numpy
+ * statement of the reference kernel within one fp16 step (rmsnorm, rotary pairs and tables,
+ * SwiGLU) or bit for bit (bias / element add); the attention against an fp64 grouped-query
+ * attention plus probes that place each probability at an element that depends on the key's
+ * index and on the query head's key/value head; the whole step (logits and the last layer's
+ * q, k, v, attention output, SwiGLU output, residual stream at 20 positions) against an
+ * independent fp64 forward of the graph.  The reference holds no fixture for these kernels
+ * that can be used without the real checkpoints, so what is pinned is the mathematics and
+ * the indexing, not a bit pattern of the reference's device.
  */
 #include "oracle.h"
 #include <math.h>
@@ -101,20 +107,20 @@ static void rope(uint16_t* buf, int heads, int D, const uint16_t* cosr, const ui
         }
 }
 
-static void attention(orc_decoder* d, int layer, int pos)
+/* gqa_attn_scores + gqa_softmax + gqa_attn_out for one query row (QW/kernels/attention.cl:43-101,
+ * 109-135, 148-186): q [n_heads*D], kc / vc [>= seq_k][n_kv_heads*D], scores scratch
+ * [n_heads][score_stride], out [n_heads*D]. */
+static void gqa_attention(const uint16_t* q, const uint16_t* kc, const uint16_t* vc, uint16_t* scores,
+                          uint16_t* out, int n_heads, int n_kv_heads, int D, int score_stride, int seq_k)
 {
-    const orc_model* m = &d->m;
-    int D = m->head_dim, kvd = m->n_kv_heads * D, nrep = m->n_heads / m->n_kv_heads;
-    int seq_k = pos + 1;
-    const uint16_t* kc = d->kc + (size_t)layer * m->max_pos * kvd;
-    const uint16_t* vc = d->vc + (size_t)layer * m->max_pos * kvd;
+    int kvd = n_kv_heads * D, nrep = n_heads / n_kv_heads;
     float scale = 1.0f / sqrtf((float)D);
-    for (int qh = 0; qh < m->n_heads; ++qh) {
+    for (int qh = 0; qh < n_heads; ++qh) {
         int kvh = qh / nrep;
-        uint16_t* sc = d->scores + (size_t)qh * m->max_pos;
+        uint16_t* sc = scores + (size_t)qh * score_stride;
         for (int tk = 0; tk < seq_k; ++tk) {                   /* gqa_attn_scores */
             float acc = 0.0f;
-            const uint16_t* qv = d->q + qh * D;
+            const uint16_t* qv = q + qh * D;
             const uint16_t* kv = kc + (size_t)tk * kvd + kvh * D;
             for (int d4 = 0; d4 < D / 4; ++d4) {
                 float t = H(qv[4 * d4]) * H(kv[4 * d4]);
@@ -139,9 +145,17 @@ static void attention(orc_decoder* d, int layer, int pos)
             float acc = 0.0f;
             for (int tk = 0; tk < seq_k; ++tk)
                 acc = fmaf(H(sc[tk]), H(vc[(size_t)tk * kvd + kvh * D + e]), acc);
-            d->attn[qh * D + e] = F(acc);
+            out[qh * D + e] = F(acc);
         }
     }
+}
+
+static void attention(orc_decoder* d, int layer, int pos)
+{
+    const orc_model* m = &d->m;
+    int kvd = m->n_kv_heads * m->head_dim;
+    gqa_attention(d->q, d->kc + (size_t)layer * m->max_pos * kvd, d->vc + (size_t)layer * m->max_pos * kvd,
+                  d->scores, d->attn, m->n_heads, m->n_kv_heads, m->head_dim, m->max_pos, pos + 1);
 }
 
 static void swiglu(uint16_t* gate, const uint16_t* up, int n)
@@ -151,6 +165,19 @@ static void swiglu(uint16_t* gate, const uint16_t* up, int n)
         float sig = 1.0f / (1.0f + orc_expf_export(-g));
         gate[i] = F((g * sig) * u);
     }
+}
+
+/* The pieces above one at a time, for the tests that pin them against independent statements
+ * (tests/test_oracle_decode.py). */
+void orc_rmsnorm(const uint16_t* x, const uint16_t* w, uint16_t* out, int cols, float eps) { rmsnorm(x, w, out, cols, eps); }
+void orc_bias_add(uint16_t* out, const uint16_t* b, int n) { bias_add(out, b, n); }
+void orc_element_add(uint16_t* a, const uint16_t* b, int n) { element_add(a, b, n); }
+void orc_rope(uint16_t* buf, int heads, int D, const uint16_t* cosr, const uint16_t* sinr) { rope(buf, heads, D, cosr, sinr); }
+void orc_swiglu(uint16_t* gate, const uint16_t* up, int n) { swiglu(gate, up, n); }
+void orc_gqa_attention(const uint16_t* q, const uint16_t* kc, const uint16_t* vc, uint16_t* scores, uint16_t* out,
+                       int n_heads, int n_kv_heads, int D, int score_stride, int seq_k)
+{
+    gqa_attention(q, kc, vc, scores, out, n_heads, n_kv_heads, D, score_stride, seq_k);
 }
 
 /* argmax_partial with NP partials of 64 lanes, then argmax_finalize
@@ -192,6 +219,21 @@ static void linear(orc_decoder* d, orc_linear_fn fn, void* ctx, int index, int N
     else orc_gemv_i8(x, d->m.w8[index], d->m.wscale[index], y, N, K, d->threads);
 }
 
+/* Rotary tables [max_pos][D], both halves of a row hold the same D/2 values
+ * (QW/src/layers/attention.cpp:147-160: fp32 pow / cos / sin, then one rounding to fp16). */
+void orc_rope_tables(int max_pos, int D, float theta, uint16_t* cosT, uint16_t* sinT)
+{
+    for (int t = 0; t < max_pos; ++t)
+        for (int i = 0; i < D / 2; ++i) {
+            float exponent = (2.0f * (float)i) / (float)D;
+            float inv_freq = powf(theta, -exponent);
+            float angle = (float)t * inv_freq;
+            uint16_t c = F(cosf(angle)), s = F(sinf(angle));
+            cosT[(size_t)t * D + i] = c; cosT[(size_t)t * D + i + D / 2] = c;
+            sinT[(size_t)t * D + i] = s; sinT[(size_t)t * D + i + D / 2] = s;
+        }
+}
+
 void* orc_decoder_new(const orc_model* m, int threads)
 {
     orc_decoder* d = (orc_decoder*)calloc(1, sizeof *d);
@@ -203,15 +245,7 @@ void* orc_decoder_new(const orc_model* m, int threads)
     d->vc = (uint16_t*)calloc(cache, 2);
     d->cosT = (uint16_t*)malloc((size_t)m->max_pos * D * 2);
     d->sinT = (uint16_t*)malloc((size_t)m->max_pos * D * 2);
-    for (int t = 0; t < m->max_pos; ++t)                      /* attention.cpp:147-160 */
-        for (int i = 0; i < D / 2; ++i) {
-            float exponent = (2.0f * (float)i) / (float)D;
-            float inv_freq = powf(m->rope_theta, -exponent);
-            float angle = (float)t * inv_freq;
-            uint16_t c = F(cosf(angle)), s = F(sinf(angle));
-            d->cosT[(size_t)t * D + i] = c; d->cosT[(size_t)t * D + i + D / 2] = c;
-            d->sinT[(size_t)t * D + i] = s; d->sinT[(size_t)t * D + i + D / 2] = s;
-        }
+    orc_rope_tables(m->max_pos, D, m->rope_theta, d->cosT, d->sinT);
     d->h = (uint16_t*)malloc(m->hidden * 2);   d->xn = (uint16_t*)malloc(m->hidden * 2);
     d->q = (uint16_t*)malloc(qd * 2);          d->k = (uint16_t*)malloc(kvd * 2);
     d->v = (uint16_t*)malloc(kvd * 2);         d->attn = (uint16_t*)malloc(qd * 2);
