@@ -66,6 +66,9 @@ _SIGNATURES = {
     "mi_decoder_buffer": (_vp, [_vp, _i]),
     "mi_argmax_f16": (_i, [_vp, _vp, _i, _i, _vp]),
     "mi_linear_argmax": (_i, [_vp, _i, _i, _vp, _vp, _vp, _i, _vp]),
+    "mi_stream_set_modes": (_i, [_vp, _i, _i]),
+    "mi_stream_read_probe": (_i, [_vp, _vp, C.c_size_t, _vp]),
+    "mi_linear_plan": (_i, [_vp, _i, _i, _i, _vp, _vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "mi_set_gemm_mode": (None, [_i]),
     "mi_set_gemv_mode": (None, [_i]),
     "mi_quantize_int8": (_i, [_vp, _i, _i, _vp, _vp]),
@@ -293,6 +296,14 @@ def argmax_f16(queue, logits, N, token_out, num_partials=32):
 def pytorch_linear_argmax(queue, N, K, x, W, logits, token_out, num_partials=32):
     """The lm_head of a greedy step: dispatch_lm_head_argmax (QW/src/model.cpp:436-482)."""
     return bool(lib().mi_linear_argmax(_q(queue), N, K, _h(x), _h(W), _h(logits), num_partials, _h(token_out)))
+
+
+def linear_plan(queue, M, N, K, x, W):
+    """(kernel, rows of x per block, slices of K) mi_linear would use; kernel 0 = GEMV rows, 1 = wide MFMA kernel,
+    2 / 3 = tile kernels."""
+    tr, ks = C.c_int(0), C.c_int(1)
+    kern = lib().mi_linear_plan(_q(queue), M, N, K, _h(x), _h(W), C.byref(tr), C.byref(ks))
+    return kern, tr.value, ks.value
 
 
 class DecoderConfig(C.Structure):

@@ -9,7 +9,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libmi_linear.so")
-SOURCES = ["runtime.hip", "gemv.hip", "gemm.hip", "argmax.hip", "decode.hip", "quantize.cpp", "bundle.cpp"]
+SOURCES = ["runtime.hip", "gemv.hip", "gemm.hip", "argmax.hip", "decode.hip", "probe.hip", "quantize.cpp", "bundle.cpp"]
 
 # -ffp-contract=off: the kernels spell every fused multiply-add as fmaf(); nothing else
 # may be fused, or results stop being bit-identical to the reference evaluation order.

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <cstdint>
 #include <cstdio>
+#include <mutex>
 
 // Error convention of the reference (QW/src/debug_utils.h:56-64): always on, stderr,
 // "ERROR: <message> (<file>:<line>)".
@@ -38,8 +39,20 @@ struct DeviceInfo {
 const DeviceInfo& device_info();
 // 0 = every GEMV evaluates the reference kernels' sum in their order (bit-exact);
 // 1 = Q4 may use the throughput kernel (same fp32 sum, other order).
-int gemv_mode();
-int gemm_mode();   // value of mi_set_gemm_mode: 0 auto, 1 rows of GEMV, others pin a GEMM kernel
+// Both are looked up for the stream a call is enqueued on: the value mi_stream_set_modes gave that
+// stream, else the process default of mi_set_gemv_mode / mi_set_gemm_mode.
+int gemv_mode(hipStream_t s);
+int gemm_mode(hipStream_t s);   // 0 auto, 1 rows of GEMV, others pin a GEMM kernel
+
+// Runs `raise` (a hipFuncSetAttribute call) once per call site and process, also when several host
+// threads arrive together; later calls return what it returned.
+#define MI_ONCE_OK(raise)                                          \
+    ([&]() -> bool {                                               \
+        static std::once_flag once_;                               \
+        static bool ok_ = false;                                   \
+        std::call_once(once_, [&] { ok_ = (raise); });             \
+        return ok_;                                                \
+    }())
 
 // M rows of x (stride K) against one W; y rows have stride N.
 struct GemvCall {
@@ -70,7 +83,7 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n);
 bool gemv_takes_norm(WeightKind kind, int K);    // GemvCall::norm_w is supported for this kind and K
 bool gemv_takes_swiglu(WeightKind kind, int K);  // EPI_SWIGLU is supported for this kind and K
 // Candidates a launch with GemvCall::am_v writes (one per wavefront of its grid), and their upper bound.
-bool gemv_takes_argmax(const GemvCall& c);       // GemvCall::am_v is supported for this call (kind, K, M, epilogue)
+bool gemv_takes_argmax(hipStream_t s, const GemvCall& c);   // GemvCall::am_v is supported for this call (kind, K, M, epilogue) on this stream
 int  gemv_argmax_slots(const GemvCall& c);
 constexpr int kGemvArgmaxMaxSlots = 8192;
 bool launch_gate_up_silu(hipStream_t s, WeightKind kind, int N, int K, const void* x,
@@ -108,6 +121,11 @@ bool launch_argmax_finish(hipStream_t s, const float* cand_v, const int* cand_i,
 bool gemm_supported(WeightKind kind, int M, int N, int K, const void* x, const void* W, const void* scale);
 // Estimated time (us) of the kernel launch_gemm would pick in mode 0.
 double gemm_estimate_us(WeightKind kind, int M, int N, int K, size_t workspace_bytes);
+// What launch_gemm would run for this call on this stream: kernel 1 = the wide kernel (tile_rows
+// rows of x per block, K in k_slices slices, `terms` fp16 terms per Q4 weight), 2 / 3 = 64 x 64 /
+// 128 x 128 tiles; kernel -1 = a mode that cannot serve this call.
+struct GemmPlan { int kernel = -1, tile_rows = 0, k_slices = 1, terms = 1; };
+GemmPlan plan_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, size_t workspace_bytes);
 // workspace: device memory that belongs to stream s (or null): the wide kernel may cut K into
 // slices and park fp32 partial sums there; calls on one stream are ordered, so they can share it.
 bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x,

@@ -961,12 +961,13 @@ void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* 
     take(d->wq, w->wq); take(d->wk, w->wk); take(d->wv, w->wv); take(d->wo, w->wo);
     take(d->wgate, w->wgate); take(d->wup, w->wup); take(d->wdown, w->wdown);
     d->embed = w->embed; d->final_norm = w->final_norm; d->lm_head = w->lm_head;
-    bool aligned = reinterpret_cast<uintptr_t>(w->final_norm) % 8 == 0;
+    // (16 bytes: the GEMV launches that carry the norm in their prologue read it in 16-byte pieces)
+    bool aligned = reinterpret_cast<uintptr_t>(w->final_norm) % 16 == 0;
     for (int l = 0; l < L; ++l)
-        aligned = aligned && reinterpret_cast<uintptr_t>(w->in_norm[l]) % 8 == 0 &&
-                  reinterpret_cast<uintptr_t>(w->post_norm[l]) % 8 == 0;
+        aligned = aligned && reinterpret_cast<uintptr_t>(w->in_norm[l]) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(w->post_norm[l]) % 16 == 0;
     if (!aligned || c.hidden % 4) {
-        MI_ERROR_FMT("mi_decoder_create: norm weights must be 8-byte aligned and hidden a multiple of 4");
+        MI_ERROR_FMT("mi_decoder_create: norm weights must be 16-byte aligned and hidden a multiple of 4");
         delete d;
         return nullptr;
     }
@@ -1198,7 +1199,8 @@ int mi_decoder_step(void* dec, void* stream) {
                                    d->rope_now, kc, vc, d->qr, d->kr, d->vr, d->attn, d->st, c.n_heads, c.n_kv_heads,
                                    c.max_pos, scale);
         } else {
-            const int at = D > 64 ? D : 64;
+            // a whole number of wavefronts: the maximum's cross-lane steps read every lane of a wavefront
+            const int at = ((D > 64 ? D : 64) + 63) & ~63;
             hipLaunchKernelGGL(rope_attention_kernel, dim3(c.n_heads), dim3(at), static_cast<size_t>(c.max_pos) * 6 + D * 6, s,
                                d->q, d->k, d->v, bq, bk, bv, d->cosT, d->sinT, kc, vc, d->qr, d->kr, d->vr, d->attn,
                                d->st, c.n_heads, c.n_kv_heads, D, c.max_pos, scale);
@@ -1306,7 +1308,16 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
             const int N2[2] = {I, I};
             if (!failed && I % 4 == 0) d->wgu[l] = stack_weights(d, s, 2, W2, N2, Hd, &failed);
         }
-        if (failed) return 0;
+        if (failed) {
+            // nothing half-built stays behind: the next prompt starts over, and no registry entry
+            // outlives the memory it names
+            if (!MI_HIP_OK(hipStreamSynchronize(s))) return 0;
+            for (void* w : d->wqkv) if (w) mi_unregister_weight(w);
+            for (void* w : d->wgu) if (w) mi_unregister_weight(w);
+            for (void* p : d->stacked_mem) { mi_unregister_weight(p); (void)hipFree(p); }
+            d->wqkv.clear(); d->wgu.clear(); d->stacked_mem.clear();
+            return 0;
+        }
         d->stacked_built = true;
     }
     if (!MI_HIP_OK(hipMemcpyAsync(tok, tokens, static_cast<size_t>(M) * 4, hipMemcpyHostToDevice, s))) return 0;
@@ -1317,12 +1328,11 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
     const unsigned gI = static_cast<unsigned>(nI / 1024 + 1 < 8192 ? nI / 1024 + 1 : 8192);
     const size_t att_lds = static_cast<size_t>(D) * 2 * (1 + kPromptTile) + static_cast<size_t>(pos0 + M) * 6;
     if (att_lds > 65536) {
-        static bool raised = false;
-        if (!raised && !MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_rows_kernel),
+        // (the most any head width and context need, so that one call serves every later shape)
+        if (!MI_ONCE_OK(MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_rows_kernel),
                                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                      D * 2 * (1 + kPromptTile) + kMaxPositions * 6)))
+                                                      256 * 2 * (1 + kPromptTile) + kMaxPositions * 6))))
             return 0;
-        raised = true;
     }
     // one block per key/value head and row where the group's scores fit the LDS of a CU (160 KB, less
     // the kernel's few static bytes)

@@ -740,12 +740,10 @@ bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, co
     }
     constexpr size_t lds_bytes = static_cast<size_t>(stages_for(KIND, TM)) * (32 * TM * 128 + w_stage_bytes(KIND));
     auto* kern = gemm_wide<TM, KIND, TERMS>;
-    static bool raised = false;
-    if (lds_bytes > 65536 && !raised) {
-        if (!MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes))) return false;
-        raised = true;
-    }
+    if (lds_bytes > 65536 &&
+        !MI_ONCE_OK(MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes))))
+        return false;
     const long total = static_cast<long>((N + kBN - 1) / kBN) * ((M + 32 * TM - 1) / (32 * TM)) * splits;
     const dim3 grid(static_cast<unsigned>(8 * ((total + 7) / 8)), 1, 1);      // see the block -> tile map in the kernel
     hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, s, static_cast<const uint16_t*>(x),
@@ -833,22 +831,19 @@ bool launch_tile(hipStream_t s, WeightKind kind, int M, int N, int K, const void
     auto* op = static_cast<uint16_t*>(out);
     constexpr size_t lds_bytes = 2u * (BM + BN) * kLd * sizeof(uint16_t);
     // more than 64 KB of LDS per block has to be asked for once per kernel
-    static bool raised_i8 = false, raised_f16 = false;
     if (kind == WK_I8) {
         auto* kern = gemm_kernel<BM, BN, WM, WN, WK_I8>;
-        if (lds_bytes > 65536 && !raised_i8) {
-            if (!MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes))) return false;
-            raised_i8 = true;
-        }
+        if (lds_bytes > 65536 &&
+            !MI_ONCE_OK(MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes))))
+            return false;
         hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, s, xp, wp, sp, op, M, N, K);
     } else {
         auto* kern = gemm_kernel<BM, BN, WM, WN, WK_F16>;
-        if (lds_bytes > 65536 && !raised_f16) {
-            if (!MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes))) return false;
-            raised_f16 = true;
-        }
+        if (lds_bytes > 65536 &&
+            !MI_ONCE_OK(MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes))))
+            return false;
         hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, s, xp, wp, sp, op, M, N, K);
     }
     return MI_HIP_OK(hipGetLastError());
@@ -898,6 +893,45 @@ double gemm_estimate_us(WeightKind kind, int M, int N, int K, size_t workspace_b
     return wide_us < tiled_us ? wide_us : tiled_us;
 }
 
+GemmPlan plan_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, size_t workspace_bytes) {
+    GemmPlan p;
+    const int mode = gemm_mode(s) == 4 && kind != WK_Q4 ? 0 : gemm_mode(s);   // mode 4 only concerns Q4 weights
+    const int cus = device_info().cus;
+    const bool wide_fits = wide_reaches(kind, M, N, K);
+    int tm = 1, splits = 1;
+    if (kind == WK_Q4) {
+        // Q4 weights have the wide kernel only; modes 3 and 11..15 pin it to one slice of K.
+        // Mode 4 feeds every weight as the single fp16 number nearest to q * scale (half the
+        // MFMAs, an error of up to 2^-12 sum |w x|); all other modes feed q * scale exactly, as
+        // two fp16 terms.
+        if (!wide_fits || mode == 2) return p;
+        p.terms = mode == 4 ? 1 : 2;
+        const bool may_slice = mode == 0 || mode == 4;
+        wide::pick_shape(WK_Q4, p.terms, M, N, K, cus, may_slice ? workspace_bytes : 0, &tm, &splits, nullptr);
+        if (mode >= 11 && mode <= 15) tm = mode - 10;
+        p.kernel = 1; p.tile_rows = 32 * tm; p.k_slices = splits;
+        return p;
+    }
+    // int8 and fp16: the wide kernel where its estimated time beats that of the 64 x 64 tiles
+    if (wide_fits && (mode == 0 || mode == 3 || (mode >= 11 && mode <= 15))) {
+        double wide_us = 0.0;
+        // modes 3 and 11..15 pin the plain kernel; slices of K are the library's own choice (mode 0)
+        wide::pick_shape(kind, 1, M, N, K, cus, mode == 0 ? workspace_bytes : 0, &tm, &splits, &wide_us);
+        if (mode >= 11) tm = mode - 10;
+        if (mode != 0 || wide_us < tiled_estimate_us(M, N, K)) {
+            p.kernel = 1; p.tile_rows = 32 * tm; p.k_slices = splits;
+            return p;
+        }
+    } else if (mode == 3 || mode >= 11) {
+        return p;
+    }
+    // 128 x 128 tiles once they fill every CU twice over (two blocks are resident per CU);
+    // below that the 64 x 64 tile spreads the work over more CUs and wins (measured).
+    const bool big = mode != 2 && M > 64 && tiles(M, N, 128, 128) >= 2L * cus;
+    p.kernel = big ? 3 : 2; p.tile_rows = big ? 128 : 64;
+    return p;
+}
+
 bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x, const void* W,
                  const void* scale, void* out, void* workspace, size_t workspace_bytes) {
     if (!gemm_supported(kind, M, N, K, x, W, scale)) {
@@ -905,50 +939,25 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
                      "without a (4-byte aligned) scale", static_cast<int>(kind), M, N, K);
         return false;
     }
-    const int mode = gemm_mode() == 4 && kind != WK_Q4 ? 0 : gemm_mode();   // mode 4 only concerns Q4 weights
-    const int cus = device_info().cus;
-    // int8 and fp16: the wide kernel where its estimated time beats that of the 64 x 64 tiles
-    const bool wide_fits = wide_reaches(kind, M, N, K);
-    if (kind == WK_Q4) {
-        // Q4 weights have the wide kernel only; modes 3 and 11..15 pin it to one slice of K.
-        // Mode 4 feeds every weight as the single fp16 number nearest to q * scale (half the
-        // MFMAs, an error of up to 2^-12 sum |w x|); all other modes feed q * scale exactly, as
-        // two fp16 terms.
-        if (!wide_fits || mode == 2) {
-            MI_ERROR_FMT("gemm: Q4 weights take the wide kernel only (mode %d, M=%d N=%d K=%d)", mode, M, N, K);
+    const size_t ws_bytes = workspace ? workspace_bytes : 0;
+    const GemmPlan p = plan_gemm(s, kind, M, N, K, ws_bytes);
+    auto* partial = static_cast<float*>(workspace);
+    switch (p.kernel) {
+        case 1: {
+            const int tm = p.tile_rows / 32;
+            if (kind == WK_Q4)
+                return p.terms == 1 ? wide::launch_any<WK_Q4, 1>(tm, s, M, N, K, x, W, scale, out, partial, ws_bytes, p.k_slices)
+                                    : wide::launch_any<WK_Q4, 2>(tm, s, M, N, K, x, W, scale, out, partial, ws_bytes, p.k_slices);
+            if (kind == WK_F16) return wide::launch_any<WK_F16, 1>(tm, s, M, N, K, x, W, scale, out, partial, ws_bytes, p.k_slices);
+            return wide::launch_any<WK_I8, 1>(tm, s, M, N, K, x, W, scale, out, partial, ws_bytes, p.k_slices);
+        }
+        case 2: return launch_tile<64, 64, 32, 32>(s, kind, M, N, K, x, W, scale, out);
+        case 3: return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);
+        default:
+            MI_ERROR_FMT("gemm: mode %d has no kernel for kind=%d M=%d N=%d K=%d (Q4 weights take the wide kernel "
+                         "only; its 32-bit offsets reach 4 GiB of x and of W)", gemm_mode(s), static_cast<int>(kind), M, N, K);
             return false;
-        }
-        const int terms = mode == 4 ? 1 : 2;
-        const bool may_slice = (mode == 0 || mode == 4) && workspace;
-        int tm = 1, splits = 1;
-        wide::pick_shape(WK_Q4, terms, M, N, K, cus, may_slice ? workspace_bytes : 0, &tm, &splits, nullptr);
-        if (mode >= 11 && mode <= 15) tm = mode - 10;
-        if (terms == 1)
-            return wide::launch_any<WK_Q4, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), workspace ? workspace_bytes : 0, splits);
-        return wide::launch_any<WK_Q4, 2>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), workspace ? workspace_bytes : 0, splits);
     }
-    if (wide_fits && (mode == 0 || mode == 3 || (mode >= 11 && mode <= 15))) {
-        double wide_us = 0.0;
-        int tm = 1, splits = 1;
-        // modes 3 and 11..15 pin the plain kernel; slices of K are the library's own choice (mode 0)
-        wide::pick_shape(kind, 1, M, N, K, cus, mode == 0 && workspace ? workspace_bytes : 0, &tm, &splits, &wide_us);
-        const double tiled_us = tiled_estimate_us(M, N, K);
-        if (mode >= 11) tm = mode - 10;
-        if (mode != 0 || wide_us < tiled_us) {
-            if (kind == WK_F16)
-                return wide::launch_any<WK_F16, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), workspace ? workspace_bytes : 0, splits);
-            return wide::launch_any<WK_I8, 1>(tm, s, M, N, K, x, W, scale, out, static_cast<float*>(workspace), workspace ? workspace_bytes : 0, splits);
-        }
-    } else if (mode == 3 || mode >= 11) {
-        MI_ERROR_FMT("gemm: mode %d asks for the wide kernel, whose 32-bit offsets do not reach M=%d N=%d K=%d",
-                     mode, M, N, K);
-        return false;
-    }
-    // 128 x 128 tiles once they fill every CU twice over (two blocks are resident per CU);
-    // below that the 64 x 64 tile spreads the work over more CUs and wins (measured).
-    if (mode != 2 && M > 64 && tiles(M, N, 128, 128) >= 2L * cus)
-        return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);
-    return launch_tile<64, 64, 32, 32>(s, kind, M, N, K, x, W, scale, out);
 }
 
 }  // namespace mi

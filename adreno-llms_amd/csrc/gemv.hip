@@ -1028,10 +1028,10 @@ bool check_call(const GemvCall& c) {
 
 // Kernels that can leave argmax candidates: the ones that keep x in registers (int8, fp16) and the
 // Q4 throughput kernel where launch_gemv_group would take it.
-bool gemv_takes_argmax(const GemvCall& c) {
+bool gemv_takes_argmax(hipStream_t s, const GemvCall& c) {
     if (c.M != 1 || c.epi != EPI_STORE) return false;
     if (c.kind == WK_Q4)
-        return !c.norm_w && gemv_mode() == 1 && pick_vl(c.kind, 1, c.N, c.K) == 4 &&
+        return !c.norm_w && gemv_mode(s) == 1 && pick_vl(c.kind, 1, c.N, c.K) == 4 &&
                (c.K == 576 || c.K == 896 || c.K == 1024 || c.K == 1536);
     return gemv_takes_norm(c.kind, c.K);
 }
@@ -1068,7 +1068,7 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
         rows += calls[i].N;
     }
     const GemvCall& c = calls[0];
-    if (c.am_v && !(n == 1 && c.am_i && c.am_np > 0 && gemv_takes_argmax(c))) {
+    if (c.am_v && !(n == 1 && c.am_i && c.am_np > 0 && gemv_takes_argmax(s, c))) {
         MI_ERROR_FMT("gemv: the fused argmax takes one segment, M = 1 and a kernel that keeps x in registers "
                      "(kind=%d K=%d)", static_cast<int>(c.kind), c.K);
         return false;
@@ -1100,7 +1100,7 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
         return vl == 2 ? launch_swiglu_vl<WK_F16, 2>(s, calls) : launch_swiglu_vl<WK_F16, 1>(s, calls);
     }
     const bool add = c.epi == EPI_ADD;
-    if (c.kind == WK_Q4 && vl == 4 && gemv_mode() == 1 && !c.norm_w) {       // (the throughput kernel has no norm)
+    if (c.kind == WK_Q4 && vl == 4 && gemv_mode(s) == 1 && !c.norm_w) {       // (the throughput kernel has no norm)
         bool taken = false;
         const bool ok = add ? launch_q4_fast<EPI_ADD>(s, calls, n, &taken) : launch_q4_fast<EPI_STORE>(s, calls, n, &taken);
         if (taken) return ok;

@@ -3,6 +3,7 @@
 #include "../../include/mi_linear.h"
 #include "common.h"
 
+#include <atomic>
 #include <cstring>
 #include <mutex>
 #include <unordered_map>
@@ -12,12 +13,16 @@ namespace {
 
 DeviceInfo g_dev;
 bool g_inited = false;
-int g_gemm_mode = 0;
-int g_gemv_mode = 1;
+// Process defaults of the two arithmetic modes; a stream can carry its own (mi_stream_set_modes),
+// so that host threads driving different streams do not change each other's arithmetic.
+std::atomic<int> g_gemm_mode{0};
+std::atomic<int> g_gemv_mode{1};
 
 // Side table W pointer -> {kind, scale, N, K}; the counterpart of s_int8_aux / s_q4_aux
-// (LF/src/utils.cpp:194-231).  The reference is single threaded and takes no lock; a
-// mutex costs nothing here and lets several host threads drive different streams.
+// (LF/src/utils.cpp:194-231).  The reference is single threaded and takes no lock; here the
+// registry, the streams' workspaces and their modes sit behind one mutex, the process-wide mode
+// defaults are atomics and one-time kernel attributes go through std::call_once, so several
+// host threads can drive different streams.
 struct Entry {
     WeightKind kind;
     const void* scale;
@@ -32,6 +37,8 @@ std::mutex g_registry_mu;
 // simply do not slice K.
 constexpr size_t kWorkspaceBytes = 16u << 20;
 std::unordered_map<hipStream_t, void*> g_workspace;
+struct StreamModes { int gemv = -1, gemm = -1; };      // -1: the process default
+std::unordered_map<hipStream_t, StreamModes> g_stream_modes;
 
 void* workspace_of(hipStream_t s) {
     std::lock_guard<std::mutex> lk(g_registry_mu);
@@ -113,17 +120,17 @@ bool fused_gemv(hipStream_t s, int n, const int* N, int K, const void* x, const 
     return launch_gemv_group(s, group, n);
 }
 
-bool linear_argmax(hipStream_t s, int N, int K, const void* x, const void* W, void* logits, const void* norm_w,
-                   float norm_eps, int num_partials, void* token_out, int* token_copy, int* counter, bool* taken) {
+bool linear_argmax_in(void* ws, hipStream_t s, int N, int K, const void* x, const void* W, void* logits,
+                      const void* norm_w, float norm_eps, int num_partials, void* token_out, int* token_copy,
+                      int* counter, bool* taken) {
     *taken = false;
     Entry e;
     if (!resolve("linear_argmax", W, N, K, &e)) return false;
-    void* ws = workspace_of(s);
     GemvCall c;
     c.x = x; c.W = W; c.scale = e.scale; c.y = logits;
     c.M = 1; c.N = N; c.K = K; c.kind = e.kind; c.epi = EPI_STORE;
     c.norm_w = norm_w; c.norm_eps = norm_eps;
-    if (!ws || !gemv_takes_argmax(c) || (norm_w && !gemv_takes_norm(e.kind, K))) return true;
+    if (!ws || !gemv_takes_argmax(s, c) || (norm_w && !gemv_takes_norm(e.kind, K))) return true;
     static_assert(kGemvArgmaxMaxSlots * 8 <= kWorkspaceBytes, "candidates fit the workspace");
     c.am_v = static_cast<float*>(ws);
     c.am_i = reinterpret_cast<int*>(c.am_v + kGemvArgmaxMaxSlots);
@@ -134,8 +141,29 @@ bool linear_argmax(hipStream_t s, int N, int K, const void* x, const void* W, vo
     return launch_gemv(s, c) && launch_argmax_finish(s, c.am_v, c.am_i, slots, N, num_partials, token_out, token_copy, counter);
 }
 
-int gemv_mode() { return g_gemv_mode; }
-int gemm_mode() { return g_gemm_mode; }
+bool linear_argmax(hipStream_t s, int N, int K, const void* x, const void* W, void* logits, const void* norm_w,
+                   float norm_eps, int num_partials, void* token_out, int* token_copy, int* counter, bool* taken) {
+    return linear_argmax_in(workspace_of(s), s, N, K, x, W, logits, norm_w, norm_eps, num_partials, token_out,
+                            token_copy, counter, taken);
+}
+
+int gemv_mode(hipStream_t s) {
+    {
+        std::lock_guard<std::mutex> lk(g_registry_mu);
+        auto it = g_stream_modes.find(s);
+        if (it != g_stream_modes.end() && it->second.gemv >= 0) return it->second.gemv;
+    }
+    return g_gemv_mode.load(std::memory_order_relaxed);
+}
+
+int gemm_mode(hipStream_t s) {
+    {
+        std::lock_guard<std::mutex> lk(g_registry_mu);
+        auto it = g_stream_modes.find(s);
+        if (it != g_stream_modes.end() && it->second.gemm >= 0) return it->second.gemm;
+    }
+    return g_gemm_mode.load(std::memory_order_relaxed);
+}
 
 }  // namespace mi
 
@@ -219,6 +247,7 @@ int mi_stream_destroy(void* s) {
             ws = it->second;
             g_workspace.erase(it);
         }
+        g_stream_modes.erase(as_stream(s));
     }
     if (ws) (void)hipFree(ws);
     return ok;
@@ -273,8 +302,19 @@ int mi_weight_kind(const void* W) {
     return lookup(W, &e) ? static_cast<int>(e.kind) : 0;
 }
 
-void mi_set_gemm_mode(int mode) { g_gemm_mode = mode; }
-void mi_set_gemv_mode(int mode) { g_gemv_mode = mode; }
+void mi_set_gemm_mode(int mode) { g_gemm_mode.store(mode, std::memory_order_relaxed); }
+void mi_set_gemv_mode(int mode) { g_gemv_mode.store(mode, std::memory_order_relaxed); }
+
+int mi_stream_set_modes(void* stream, int gemv_mode, int gemm_mode) {
+    if (gemv_mode < -1 || gemv_mode > 1 || gemm_mode < -1) {
+        MI_ERROR_FMT("mi_stream_set_modes: bad argument (gemv_mode=%d gemm_mode=%d)", gemv_mode, gemm_mode);
+        return 0;
+    }
+    std::lock_guard<std::mutex> lk(g_registry_mu);
+    if (gemv_mode < 0 && gemm_mode < 0) g_stream_modes.erase(as_stream(stream));
+    else g_stream_modes[as_stream(stream)] = StreamModes{gemv_mode, gemm_mode};
+    return 1;
+}
 
 // ---- hot path --------------------------------------------------------------------
 
@@ -283,8 +323,9 @@ void mi_set_gemv_mode(int mode) { g_gemv_mode = mode; }
 // do batches below 16 rows while that is estimated to be faster (each GEMV row streams W again:
 // about bytes / 6.6 TB/s, or 1 us when W stays in the caches).
 static bool takes_gemm(hipStream_t s, const Entry& e, int M, int N, int K, const void* x, const void* W) {
-    if (M < 2 || g_gemm_mode == 1 || !gemm_supported(e.kind, M, N, K, x, W, e.scale)) return false;
-    if (M >= 16 || g_gemm_mode != 0) return true;
+    const int mode = gemm_mode(s);
+    if (M < 2 || mode == 1 || !gemm_supported(e.kind, M, N, K, x, W, e.scale)) return false;
+    if (M >= 16 || mode != 0) return true;
     const double w_bytes = static_cast<double>(N) * K * (e.kind == WK_F16 ? 2.0 : e.kind == WK_I8 ? 1.0 : 0.5625);
     const double row_us = w_bytes / 6.6e6 > 1.0 ? w_bytes / 6.6e6 : 1.0;
     return gemm_estimate_us(e.kind, M, N, K, workspace_of(s) ? kWorkspaceBytes : 0) < 2.5 + M * row_us;
@@ -305,6 +346,19 @@ int mi_linear(void* stream, int M, int N, int K, const void* x, const void* W, v
     c.x = x; c.W = W; c.scale = e.scale; c.y = out;
     c.M = M; c.N = N; c.K = K; c.kind = e.kind; c.epi = EPI_STORE;
     return launch_gemv(as_stream(stream), c) ? 1 : 0;
+}
+
+int mi_linear_plan(void* stream, int M, int N, int K, const void* x, const void* W, int* tile_rows, int* k_slices) {
+    if (!ensure_init()) return -1;
+    Entry e;
+    if (M <= 0 || N <= 0 || K <= 0 || !x || !W || !resolve("mi_linear_plan", W, N, K, &e)) return -1;
+    if (tile_rows) *tile_rows = 0;
+    if (k_slices) *k_slices = 1;
+    if (!takes_gemm(as_stream(stream), e, M, N, K, x, W)) return 0;
+    const GemmPlan p = plan_gemm(as_stream(stream), e.kind, M, N, K, workspace_of(as_stream(stream)) ? kWorkspaceBytes : 0);
+    if (tile_rows) *tile_rows = p.tile_rows;
+    if (k_slices) *k_slices = p.k_slices;
+    return p.kernel;
 }
 
 int mi_argmax_f16(void* stream, const void* logits, int N, int num_partials, void* token_out) {

@@ -50,16 +50,40 @@ def algo_bytes_f16(N, K):
     return 2 * N * K + 2 * K + 2 * N
 
 
-def time_region(mil, queue, fn, reps):
+def time_region(mil, queue, fn, reps, samples=1):
+    """ms per call of fn: `samples` regions of `reps` calls each, bracketed by HIP events on the
+    launch stream; the median region (samples = 1: that one region)."""
     e0, e1 = mil.Event(), mil.Event()
-    queue.finish()
-    e0.record(queue)
-    for _ in range(reps):
-        fn()
-    e1.record(queue)
-    e1.synchronize()
-    queue.finish()
-    return e0.elapsed_ms(e1) / reps
+    got = []
+    for _ in range(samples):
+        queue.finish()
+        e0.record(queue)
+        for _ in range(reps):
+            fn()
+        e1.record(queue)
+        e1.synchronize()
+        queue.finish()
+        got.append(e0.elapsed_ms(e1) / reps)
+    got.sort()
+    return got[len(got) // 2]
+
+
+def host_cpu():
+    """(model string, cores this process may run on, cores online) of the host."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        allowed = len(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = os.cpu_count()
+    return model, allowed, os.cpu_count()
 
 
 def main():
@@ -94,7 +118,7 @@ def main():
     # other as they do in the model (the attention and SwiGLU kernels that sit between the
     # projections are not part of this path and are left out): hidden -> q,k,v ; q -> o ;
     # o -> gate,up ; gate -> down ; down is the next layer's hidden ; last hidden -> lm_head.
-    keep, calls = [], []
+    keep, calls, call_family = [], [], []
     x_h = mil.Buffer.from_host(mil.synth_normal_f16(1, 1.0, (H,)))
     x_i = mil.Buffer.from_host(mil.synth_normal_f16(2, 1.0, (INTER,)))
     outs = {n: mil.Buffer(N * 2) for n, N, _ in LAYER_SHAPES}
@@ -114,9 +138,12 @@ def main():
             src = {"q": cur, "k": cur, "v": cur, "o": outs["q"], "gate": outs["o"], "up": outs["o"],
                    "down": outs["gate"]}[name]
             calls.append((1, N, K, src, qb, nxt if name == "down" else outs[name]))
+            call_family.append({"q": "qkv", "k": "qkv", "v": "qkv", "o": "o", "gate": "gate_up", "up": "gate_up",
+                                "down": "down"}[name])
             sweep_bytes += N * K + 2 * N
     lm_q, lm_s, lm_host = make_i8(7, VOCAB, H)
     calls.append((1, VOCAB, H, hidden[LAYERS % 2], lm_q, logits))
+    call_family.append("lm_head")
     sweep_bytes += VOCAB * H + 2 * VOCAB
     assert sweep_bytes == 494873344, sweep_bytes
     call_arr = mil.make_calls(calls)
@@ -141,6 +168,9 @@ def main():
 
     launch_mode = "hip_graph" if ms_graph < ms_stream else "stream"
     ms_step = min(ms_graph, ms_stream)
+    # the same step as the median of ten shorter regions (the headline is the mean over all K steps)
+    per = max(1, args.steps // 10)
+    ms_step_median = time_region(mil, queue, sweep_stream if launch_mode == "stream" else graph.launch, per, 10)
     value = sweep_bytes / (ms_step * 1e-3) / 1e9
 
     # ---- roofline of the dominant kernel: lm_head int8 GEMV, cold ---------------------------
@@ -155,16 +185,64 @@ def main():
     lm_calls = mil.make_calls([(1, VOCAB, H, x_h, copies[i % 3][0], logits) for i in range(30)])
     for _ in range(2):
         mil.linear_batch(queue, lm_calls)
-    ms_lm = time_region(mil, queue, lambda: mil.linear_batch(queue, lm_calls), 10) / 30
+    ms_lm = time_region(mil, queue, lambda: mil.linear_batch(queue, lm_calls), 2, 9) / 30
     lm_bytes = algo_bytes_i8(VOCAB, H)
     achieved = lm_bytes / (ms_lm * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "gemv int8 K=896 (lm_head, N=151936)", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": LM_HEAD_I8_TRAFFIC_BYTES, "us_per_launch": round(ms_lm * 1e3, 2), "bytes_per_launch": lm_bytes}
+                "traffic": LM_HEAD_I8_TRAFFIC_BYTES,
+                "traffic_source": "constant from profiles/gemv_int8_lm_head_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE, "
+                                  "WRITE_SIZE of this kernel, scaled by a copy of known size); not measured by this run",
+                "us_per_launch": round(ms_lm * 1e3, 2), "bytes_per_launch": lm_bytes,
+                "timing": "median of 9 regions of 60 launches, HIP events on the launch stream, weights rotate through "
+                          "3 copies (408 MB) so every launch streams from HBM"}
 
     # ---- per-config detail -------------------------------------------------------------------
     detail = {"decode_step_us_stream": round(ms_stream * 1e3, 1), "decode_step_us_graph": None if args.no_graph else round(ms_graph * 1e3, 1),
-              "setup_s": round(setup_s, 1)}
+              "decode_step_us_median_of_10_regions": round(ms_step_median * 1e3, 1), "setup_s": round(setup_s, 1)}
+
+    # ---- the launches the step's time goes to: each family of launches timed by leaving it out ----
+    # (a launch inside a chain of dependent launches cannot be bracketed by events without changing
+    # the chain; the sweep without one family, weights as cold as in the full sweep, can)
+    if not args.no_detail:
+        fam_rows = {"qkv": H + 2 * KV, "o": H, "gate_up": 2 * INTER, "down": H, "lm_head": VOCAB}
+        fam_k = {"qkv": H, "o": H, "gate_up": H, "down": INTER, "lm_head": H}
+        by_time = []
+        for fam in ("gate_up", "down", "qkv", "o", "lm_head"):
+            sub = mil.make_calls([c for c, f in zip(calls, call_family) if f != fam])
+            run = lambda: mil.linear_batch(queue, sub)
+            if not args.no_graph:
+                with mil.Graph(queue) as gsub:
+                    mil.linear_batch(queue, sub)
+                run = gsub.launch
+            for _ in range(5):
+                run()
+            ms_without = time_region(mil, queue, run, per, 10)
+            n_launch = 1 if fam == "lm_head" else LAYERS
+            us = max(ms_step_median - ms_without, 1e-6) * 1e3 / n_launch
+            nbytes = fam_rows[fam] * fam_k[fam] + 4 * fam_rows[fam] + 2 * fam_k[fam]
+            by_time.append({"kernel": f"gemv int8 {fam} ({fam_rows[fam]} rows x {fam_k[fam]}), one launch",
+                            "launches_per_step": n_launch, "bytes_per_launch": nbytes, "us_per_launch": round(us, 2),
+                            "achieved": round(nbytes / us / 1e3, 1), "unit": "GB/s", "peak": HBM_PEAK_GBS,
+                            "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                            "share_of_step": round(us * n_launch / (ms_step_median * 1e3), 3)})
+        detail["roofline_by_time"] = {
+            "how": "time of the sweep minus time of the sweep without that family of launches (median of 10 regions each), "
+                   "per launch; bound hbm; the launches are latency-bound, see frac",
+            "kernels": by_time}
+
+    # ---- what a pure reader gets: the practical ceiling beside the 8 TB/s peak ------------------
+    # (the reference's gemv_stream_buf probe, QW/kernels/gemv_m1.cl:105-131); the three lm_head copies
+    # are contiguous enough for this purpose: each launch reads one copy, rotating
+    def read_probe(nbytes):
+        fn = lambda: [mil.lib().mi_stream_read_probe(queue.handle, copies[i % 3][0].ptr, nbytes, None) for i in range(30)]
+        fn()
+        ms = time_region(mil, queue, fn, 2, 9) / 30
+        return {"bytes": nbytes, "us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                "frac_hbm": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    detail["read_probe_int8_lm_head_bytes"] = read_probe(VOCAB * H)
+    detail["read_probe_q4_lm_head_bytes"] = read_probe(algo_bytes_q4(VOCAB, H) // 16 * 16)
+    roofline["frac_of_read_probe"] = round(detail["read_probe_int8_lm_head_bytes"]["us"] / roofline["us_per_launch"], 4)
     if not args.no_detail:
         def cold_gemv(kind, N, K, reps_pool):
             """us per launch over a pool of distinct weights larger than the last-level cache."""
@@ -192,16 +270,16 @@ def main():
             yb = mil.Buffer(N * 2)
             arr = mil.make_calls([(1, N, K, xb, pool[i % npool][0], yb) for i in range(max(npool, 32))])
             mil.linear_batch(queue, arr)
-            ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 5) / len(arr)
+            ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 1, 7) / len(arr)
             if not args.no_graph:
                 with mil.Graph(queue) as g:
                     mil.linear_batch(queue, arr)
                 g.launch()
-                ms = min(ms, time_region(mil, queue, g.launch, 5) / len(arr))
+                ms = min(ms, time_region(mil, queue, g.launch, 1, 7) / len(arr))
             # warm: the same weights every launch (they stay in the last-level cache)
             warm = mil.make_calls([(1, N, K, xb, pool[0][0], yb)] * 32)
             mil.linear_batch(queue, warm)
-            ms_warm = time_region(mil, queue, lambda: mil.linear_batch(queue, warm), 5) / 32
+            ms_warm = time_region(mil, queue, lambda: mil.linear_batch(queue, warm), 1, 7) / 32
             for wb, _ in pool:
                 mil.nnopt_unregister_weight(wb)
             return {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
@@ -212,12 +290,21 @@ def main():
         detail["c2_int8_gemv_4864x896"] = cold_gemv("i8", INTER, H, 140)
         detail["c2_int8_gemv_896x4864"] = cold_gemv("i8", H, INTER, 140)
         detail["c3_q4_gemv_151936x896"] = cold_gemv("q4", VOCAB, H, 4)
+        detail["c3_q4_gemv_151936x896"]["gemv_mode"] = 1      # the throughput kernel: within 1e-3 / cosine 0.9999 of the oracle
+        mil.lib().mi_set_gemv_mode(0)
+        try:
+            detail["c3_q4_gemv_151936x896_exact_order"] = cold_gemv("q4", VOCAB, H, 4)
+            detail["c3_q4_gemv_151936x896_exact_order"]["gemv_mode"] = 0   # bit-identical to the oracle
+        finally:
+            mil.lib().mi_set_gemv_mode(1)
+        for key in ("c3_q4_gemv_151936x896", "c3_q4_gemv_151936x896_exact_order"):
+            detail[key]["frac_of_read_probe"] = round(detail["read_probe_q4_lm_head_bytes"]["us"] / detail[key]["us"], 4)
         detail["c3_int8_gemv_151936x896"] = {"us": roofline["us_per_launch"], "GBps": roofline["achieved"],
                                              "frac_hbm": roofline["frac"], "bytes": lm_bytes}
         # the fused epilogues at the boundary (int8, warm): residual add, gate/up + SwiGLU, w3 + silu_mul
         def fused_us(fn, n=32):
             fn()
-            return round(time_region(mil, queue, lambda: [fn() for _ in range(n)], 5) / n * 1e3, 2)
+            return round(time_region(mil, queue, lambda: [fn() for _ in range(n)], 1, 7) / n * 1e3, 2)
         wq = {}
         for name, (N, K) in (("down", (H, INTER)), ("gate", (INTER, H)), ("up", (INTER, H))):
             a_, b_ = mil.quantize_int8(mil.synth_normal_f16(300 + len(wq), 0.02, (N, K)))
@@ -241,7 +328,7 @@ def main():
                 assert mil.pytorch_linear_argmax(queue, VOCAB, H, x_h, copies[i % 3][0], logits, token)
 
         lm_head_argmax()
-        detail["c4_lm_head_int8_plus_argmax"] = {"us": round(time_region(mil, queue, lm_head_argmax, 5) / 30 * 1e3, 2)}
+        detail["c4_lm_head_int8_plus_argmax"] = {"us": round(time_region(mil, queue, lm_head_argmax, 1, 7) / 30 * 1e3, 2)}
 
     # ---- config 4, whole step: every kernel of a greedy decode step on the device -----------
     if not args.no_detail and not args.no_graph:
@@ -268,7 +355,7 @@ def main():
             assert dec.step(queue)
         for _ in range(8):
             step_graph.launch()
-        ms_tok = time_region(mil, queue, step_graph.launch, 64)
+        ms_tok = time_region(mil, queue, step_graph.launch, 8, 9)
         pos_after, _ = dec.read(queue)
         detail["c4_whole_decode_step_on_device"] = {
             "us_per_token": round(ms_tok * 1e3, 1), "tokens_per_s": round(1e3 / ms_tok, 1),
@@ -298,7 +385,7 @@ def main():
             assert dec.step(queue)
         for _ in range(8):
             step_graph_q4.launch()
-        ms_tok = time_region(mil, queue, step_graph_q4.launch, 64)
+        ms_tok = time_region(mil, queue, step_graph_q4.launch, 8, 9)
         detail["c4_whole_decode_step_on_device_q4_weights"] = {
             "us_per_token": round(ms_tok * 1e3, 1), "tokens_per_s": round(1e3 / ms_tok, 1), "launch": "hip_graph"}
         dec.close()
@@ -319,7 +406,7 @@ def main():
                 ob = mil.Buffer(M * N * 2)
                 arr = mil.make_calls([(M, N, K, xb, wb, ob)] * 20)
                 mil.linear_batch(queue, arr)
-                ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 5) / 20
+                ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 1, 9) / 20
                 flop = 2.0 * M * N * K
                 nbytes = 2 * M * K + N * K + 2 * N + 2 * M * N
                 detail[f"c5_int8_gemm_M{M}_N{N}_K{K}"] = {
@@ -333,7 +420,7 @@ def main():
         ob = mil.Buffer(16 * VOCAB * 2)
         arr = mil.make_calls([(16, VOCAB, H, xb, copies[i % 3][0], ob) for i in range(9)])
         mil.linear_batch(queue, arr)
-        ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 5) / 9
+        ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 1, 9) / 9
         nbytes = VOCAB * H + 2 * VOCAB + 2 * 16 * H + 2 * 16 * VOCAB
         detail[f"c5_int8_gemm_M16_N{VOCAB}_K{H}"] = {
             "us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
@@ -346,7 +433,7 @@ def main():
             ob = mil.Buffer(M * N * 2)
             arr = mil.make_calls([(M, N, K, xb, wb, ob)] * 20)
             mil.linear_batch(queue, arr)
-            ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 5) / 20
+            ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 1, 9) / 20
             flop = 2.0 * M * N * K
             detail[f"c5_fp16_gemm_M{M}_N{N}_K{K}"] = {
                 "us": round(ms * 1e3, 2), "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 1),
@@ -364,7 +451,7 @@ def main():
                 mil.lib().mi_set_gemm_mode(mode)
                 try:
                     mil.linear_batch(queue, arr)
-                    ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 5) / 20
+                    ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 1, 9) / 20
                 finally:
                     mil.lib().mi_set_gemm_mode(0)
                 flop = 2.0 * M * N * K
@@ -382,7 +469,7 @@ def main():
         for M in (64, 512, 2048):
             ids = [int(t) for t in np.random.default_rng(M).integers(0, VOCAB, M)]
             assert big.prefill(queue, ids)
-            ms = time_region(mil, queue, lambda: big.prefill(queue, ids), 3)
+            ms = time_region(mil, queue, lambda: big.prefill(queue, ids), 1, 3)
             detail[f"c5_whole_prompt_on_device_M{M}"] = {
                 "ms": round(ms, 3), "prompt_tokens_per_s": round(M / ms * 1e3, 0),
                 "vs_single_token_steps": round(M * ms_tok / ms, 1)}
@@ -435,7 +522,9 @@ def main():
             for name, fn in cases.items():
                 detail["cpu_port"][name] = {"us_all_cores": cpu_us(lambda: fn(threads)),
                                             "us_one_core": cpu_us(lambda: fn(1))}
+        cpu_model, cpu_allowed, cpu_online = host_cpu()
         cpu = {"value": round(sample_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+               "cpu_model": cpu_model, "cores_in_affinity_mask": cpu_allowed, "cores_online": cpu_online,
                "sample": f"{reps} x (layer 0's 7 int8 GEMVs + the lm_head GEMV), {sample_bytes} algorithmic "
                          f"bytes in {dt:.1f} s, OpenMP over rows"}
 

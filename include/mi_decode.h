@@ -28,7 +28,7 @@ typedef struct mi_decoder_config {
 /* Device pointers, caller-owned, alive as long as the decoder.  Norm weights and biases are fp16
  * vectors; embed is fp16 [vocab, hidden]; projection weights are fp16 [N, K] or quantised and
  * registered (mi_register_int8_weight / mi_register_q4_weight).  Arrays have n_layers entries.
- * Norm weights must be 8-byte aligned, projection weights 16-byte aligned (anything from mi_malloc is). */
+ * Norm weights and projection weights must be 16-byte aligned (anything from mi_malloc is). */
 typedef struct mi_decoder_weights {
     const void* embed;
     const void* final_norm;

@@ -173,6 +173,28 @@ void mi_set_gemm_mode(int mode);
  * accept (cosine per layer), not bit-identical. */
 void mi_set_gemv_mode(int mode);
 
+/* The two modes above are process defaults.  This gives one stream its own: every later call
+ * enqueued on `stream` computes in gemv_mode / gemm_mode whatever the defaults are, so host
+ * threads that drive different streams cannot change each other's arithmetic.  -1 for a mode =
+ * follow the process default; (-1, -1) forgets the stream.  No counterpart in the reference (its
+ * host is single threaded and has one arithmetic). */
+int mi_stream_set_modes(void* stream, int gemv_mode, int gemm_mode);
+
+/* What mi_linear(stream, M, N, K, x, W, out) would run, without running it: 0 = GEMV (once per
+ * row of x), 1 = the wide MFMA kernel with *tile_rows rows of x per block and K cut into
+ * *k_slices slices (more than one slice: fp32 partial sums in the stream's workspace and a
+ * reduction launch), 2 / 3 = the 64 x 64 / 128 x 128 tile kernel, -1 = bad arguments.  For
+ * tests and tuning; tile_rows and k_slices may be NULL. */
+int mi_linear_plan(void* stream, int M, int N, int K, const void* x, const void* W, int* tile_rows, int* k_slices);
+
+/* Streaming-read probe: reads `bytes` (a multiple of 16 is read; src 16-byte aligned) from src
+ * with the GEMV kernels' access pattern and grid and does nothing with them; timed by the caller,
+ * it gives the rate the memory system sustains for a pure reader, the practical ceiling beside
+ * the published peak.  The reference ships the same probe for its GEMVs (gemv_stream_buf,
+ * QW/kernels/gemv_m1.cl:105-131, driven by QW/src/main.cpp:27-154).  sink: 4 bytes of device
+ * memory or NULL (never written for ordinary data). */
+int mi_stream_read_probe(void* stream, const void* src, size_t bytes, void* sink);
+
 /* ---- offline tools (host) -------------------------------------------------------- */
 
 /* quantize_row_symmetric over N rows (LF/scripts/quantize_weights.py:53-57). */

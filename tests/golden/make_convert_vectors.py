@@ -100,13 +100,13 @@ def main():
 
     for tag, inp, mid in (("single", os.path.join(OUT, "single.safetensors"), "synthetic/single"),
                           ("sharded", shard_dir, None)):
-        dst = os.path.join(OUT, f"{tag}.out")
+        dst = os.path.join(OUT, f"{tag}.bundle")
         subprocess.check_call([sys.executable, REF, "--input", inp, "--output-dir", dst]
                               + (["--model-id", mid] if mid else []))
 
     # --check-against: a reference meta with a missing tensor, an extra one, a changed shape, offset,
     # size and element count, and another total; the tool's report is the fixture
-    with open(os.path.join(OUT, "single.out", "model.fp16.meta.json")) as f:
+    with open(os.path.join(OUT, "single.bundle", "model.fp16.meta.json")) as f:
         meta = json.load(f)
     t = meta["tensors"]
     del t["extras.u8"]
@@ -119,7 +119,7 @@ def main():
     other = os.path.join(OUT, "single.other.meta.json")
     with open(other, "w") as f:
         json.dump(meta, f, indent=2)
-    for tag, against in (("mismatch", other), ("match", os.path.join(OUT, "single.out", "model.fp16.meta.json"))):
+    for tag, against in (("mismatch", other), ("match", os.path.join(OUT, "single.bundle", "model.fp16.meta.json"))):
         r = subprocess.run([sys.executable, REF, "--input", os.path.join(OUT, "single.safetensors"),
                             "--check-against", against], capture_output=True, text=True)
         text = r.stdout.replace(OUT + os.sep, "")            # paths relative to the fixture folder

@@ -28,8 +28,8 @@ def run(inp, **kw):
 def test_bundle_is_byte_identical_to_the_reference_tools_output(tmp_path, tag, inp, model_id):
     rc, text = run(os.path.join(G, inp), output_dir=str(tmp_path), model_id=model_id)
     assert rc == 0
-    want_bin = open(os.path.join(G, f"{tag}.out", "model.fp16.bin"), "rb").read()
-    want_meta = open(os.path.join(G, f"{tag}.out", "model.fp16.meta.json")).read()
+    want_bin = open(os.path.join(G, f"{tag}.bundle", "model.fp16.bin"), "rb").read()
+    want_meta = open(os.path.join(G, f"{tag}.bundle", "model.fp16.meta.json")).read()
     assert open(tmp_path / "model.fp16.bin", "rb").read() == want_bin
     assert open(tmp_path / "model.fp16.meta.json").read() == want_meta
     meta = json.loads(want_meta)
@@ -51,12 +51,12 @@ def test_a_directory_without_index_takes_every_safetensors_file(tmp_path):
     rc, _ = run(str(d), output_dir=str(tmp_path / "o"))
     assert rc == 0
     assert open(tmp_path / "o" / "model.fp16.bin", "rb").read() == \
-        open(os.path.join(G, "sharded.out", "model.fp16.bin"), "rb").read()
+        open(os.path.join(G, "sharded.bundle", "model.fp16.bin"), "rb").read()
     assert json.load(open(tmp_path / "o" / "model.fp16.meta.json"))["model_id"] == "noindex"
 
 
 @pytest.mark.parametrize("tag,against", [("mismatch", "single.other.meta.json"),
-                                         ("match", os.path.join("single.out", "model.fp16.meta.json"))])
+                                         ("match", os.path.join("single.bundle", "model.fp16.meta.json"))])
 def test_check_against_report_is_the_reference_tools(tmp_path, tag, against):
     want = open(os.path.join(G, f"single.check_{tag}.txt")).read()
     want_rc, want_text = int(want.split("\n", 1)[0].split()[1]), want.split("\n", 1)[1]

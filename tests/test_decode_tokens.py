@@ -193,6 +193,11 @@ def test_smollm_widths_fp16_and_q4_weights_on_device(kind):
     ("wide_heads_two_tiles", dict(hidden=1024, inter=1536, n_heads=8, n_kv_heads=2, head_dim=128, n_layers=1,
                                   vocab=2048, max_pos=141, rms_eps=1e-6, rope_theta=500000.0), 140),
     ("three_tiles", dict(SMOL, max_pos=267, n_layers=1), 266),
+    # head widths that are no whole number of wavefronts (the per-head kernel's block is rounded up to one)
+    ("head_dim_80", dict(hidden=640, inter=1024, n_heads=8, n_kv_heads=2, head_dim=80, n_layers=2, vocab=1024,
+                         max_pos=100, rms_eps=1e-6, rope_theta=10000.0), 90),
+    ("head_dim_96", dict(hidden=576, inter=1536, n_heads=6, n_kv_heads=3, head_dim=96, n_layers=1, vocab=1024,
+                         max_pos=70, rms_eps=1e-5, rope_theta=100000.0), 66),
 ])
 def test_device_step_other_geometries(name, cfg, steps):
     """Long sequences, 128-wide heads and a cache filled to its last row: tokens and the last logits

@@ -33,11 +33,11 @@ def _ulp_apart(a_u16, b_u16):
     return np.abs(a - b) / step
 
 
-def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0):
+def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0, plan=None):
     """tile is the mi_set_gemm_mode value: 0 = the library's own choice, 1 = rows of GEMV,
     2 = the 64 x 64 MFMA kernel, 3 = the wide kernel with its own choice of rows of x per
     block, 4 = Q4 weights rounded to fp16 once, 11..15 = the wide kernel with 32, 64, .. 160 rows
-    of x per block."""
+    of x per block.  plan: a list that receives (kernel, rows of x per block, slices of K) of the call."""
     xb, wb = mil.Buffer.from_host(X), mil.Buffer.from_host(W_host)
     sb = mil.Buffer.from_host(scale_host) if scale_host is not None else None
     if kind == "i8":
@@ -49,6 +49,8 @@ def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0):
     ob = mil.Buffer.from_host(guard)
     mil.lib().mi_set_gemm_mode(tile)
     try:
+        if plan is not None:
+            plan.append(mil.linear_plan(queue, M, N, K, xb, wb))
         assert mil.pytorch_linear(queue, M, N, K, xb, wb, ob.ptr + 2 * pad)
         queue.finish()
     finally:
@@ -297,18 +299,27 @@ def test_q4_gemm_repeats_identically(queue, tile):
     mil.nnopt_unregister_weight(wb)
 
 
-def test_q4_prefill_size_rows_sampled(queue):
-    M, N, K = 2048, 4864, 896
-    W, X = synth_w(1920, N, K), synth_x(1921, M, K)
+SAMPLED_ROWS = [0, 1, 31, 32, 63, 64, 127, 128, 159, 160, 255, 256, 1000, 1023, 1024, 2046, 2047]
+
+
+@pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864)])
+def test_q4_prefill_size_rows_sampled(queue, N, K):
+    """Config 5 at M = 2048 with Q4 weights, both shapes, as bench.py times them (at N = 896 the library
+    cuts K into slices: fp32 partial sums and a reduction launch)."""
+    M = 2048
+    W, X = synth_w(1920 + N, N, K), synth_x(1921 + N, M, K)
     p, s = mil.quantize_q4(W)
-    got = _gemm(queue, M, N, K, X, p, s, "q4")
-    for r in [0, 1, 31, 32, 159, 160, 1000, 1023, 1024, 2046, 2047]:
+    plan = []
+    got = _gemm(queue, M, N, K, X, p, s, "q4", plan=plan)
+    assert plan[0][0] == 1 and (plan[0][2] > 1) == (N == 896), plan
+    for r in SAMPLED_ROWS:
         want = O.gemv_q4(X[r], p, s.view(np.uint16))
         assert _ulp_apart(got[r], want).max() <= 1, f"row {r}"
     X2 = X.copy()
     X2[5] = X[5] * np.float16(2.0)
     got2 = _gemm(queue, M, N, K, X2, p, s, "q4")
-    assert np.array_equal(got2[5].view(np.float16), got[5].view(np.float16) * np.float16(2.0))
+    normal = np.abs(got[5].view(np.float16)) >= np.float16(2.0 ** -13)      # (a subnormal fp16 output has fewer bits)
+    assert np.array_equal(got2[5].view(np.float16)[normal], (got[5].view(np.float16) * np.float16(2.0))[normal])
     assert np.array_equal(got2[6], got[6])
 
 
@@ -319,7 +330,7 @@ def test_fp16_prefill_size_rows_sampled(queue):
         M = 2048
         W, X = synth_w(2920 + N, N, K), synth_x(2921 + N, M, K)
         got = _gemm(queue, M, N, K, X, W, None, "f16")
-        for r in [0, 1, 31, 32, 159, 160, 1000, 1023, 1024, 2046, 2047]:
+        for r in SAMPLED_ROWS:
             want = O.gemv_f16(X[r], W)
             assert _ulp_apart(got[r], want).max() <= 1, f"N={N} K={K} row {r}"
         X2 = X.copy()
@@ -330,22 +341,31 @@ def test_fp16_prefill_size_rows_sampled(queue):
         assert np.array_equal(got2[6], got[6])
 
 
-def test_prefill_size_rows_sampled(queue):
-    """Config 5 at M = 2048: every sampled row of out equals the GEMV of that row of x."""
-    M, N, K = 2048, 4864, 896
-    W, X = synth_w(920, N, K), synth_x(921, M, K)
+@pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864)])
+def test_prefill_size_rows_sampled(queue, N, K):
+    """Config 5 at M = 2048, both shapes, the kernels bench.py times: every sampled row of out equals the
+    GEMV of that row of x.  At N = 896 the tiles are too few for the chip, so the library cuts K into
+    slices (fp32 partial sums in the stream's workspace, then the reduction launch): asserted."""
+    M = 2048
+    W, X = synth_w(920 + N, N, K), synth_x(921 + N, M, K)
     q, s = mil.quantize_int8(W)
-    got = _gemm(queue, M, N, K, X, q, s, "i8")
-    rows = np.array([0, 1, 31, 32, 127, 128, 255, 256, 1000, 1023, 1024, 2046, 2047])
-    for r in rows:
+    plan = []
+    got = _gemm(queue, M, N, K, X, q, s, "i8", plan=plan)
+    assert plan[0][0] == 1 and (plan[0][2] > 1) == (N == 896), plan
+    for r in SAMPLED_ROWS:
         want = O.gemv_i8(X[r], q, s.view(np.uint16))
         assert _ulp_apart(got[r], want).max() <= 1, f"row {r}"
     # linearity in x: scaling a row of x by 2 scales the output row by 2 exactly
     X2 = X.copy()
     X2[5] = X[5] * np.float16(2.0)
     got2 = _gemm(queue, M, N, K, X2, q, s, "i8")
-    assert np.array_equal(got2[5].view(np.float16), got[5].view(np.float16) * np.float16(2.0))
+    normal = np.abs(got[5].view(np.float16)) >= np.float16(2.0 ** -13)
+    assert np.array_equal(got2[5].view(np.float16)[normal], (got[5].view(np.float16) * np.float16(2.0))[normal])
     assert np.array_equal(got2[6], got[6])
+    # every row, not only the sampled ones, against the rows-of-GEMV mode of the same entry point
+    rows = _gemm(queue, M, N, K, X, q, s, "i8", tile=1)
+    assert _ulp_apart(got, rows).max() <= 1
+    assert np.mean(got == rows) > 0.99
 
 
 def test_batched_gemv_mode_stays_bit_exact(queue):
@@ -386,3 +406,35 @@ def test_gemm_random_shapes(queue, kind):
             assert_tolerance(got.view(np.float16), want.view(np.float16))
             if not (kind == "q4" and tile == 0):
                 assert _ulp_apart(got, want).max() <= 1, (M, N, K, tile)
+
+
+def test_modes_belong_to_the_stream_that_set_them(queue):
+    """mi_stream_set_modes: a stream's own gemm / gemv mode holds whatever the process default says,
+    and another stream keeps following the default."""
+    L = mil.lib()
+    M, N, K = 64, 896, 896
+    W, X = synth_w(4100, N, K), synth_x(4101, M, K)
+    q, s = mil.quantize_int8(W)
+    xb, wb, sb = mil.Buffer.from_host(X), mil.Buffer.from_host(q), mil.Buffer.from_host(s)
+    assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+    other = mil.Queue()
+    try:
+        assert mil.linear_plan(queue, M, N, K, xb, wb)[0] > 0 and mil.linear_plan(other, M, N, K, xb, wb)[0] > 0
+        assert L.mi_stream_set_modes(other.handle, -1, 1) == 1          # rows of GEMV on `other` only
+        assert mil.linear_plan(other, M, N, K, xb, wb)[0] == 0
+        assert mil.linear_plan(queue, M, N, K, xb, wb)[0] > 0
+        a, b = mil.Buffer(M * N * 2), mil.Buffer(M * N * 2)
+        assert mil.pytorch_linear(other, M, N, K, xb, wb, a)
+        other.finish()
+        assert np.array_equal(a.read(np.uint16, (M, N)), O.gemm_i8(X, q, s.view(np.uint16)))   # bit-exact rows
+        L.mi_set_gemm_mode(1)                                            # the default changes ...
+        assert L.mi_stream_set_modes(other.handle, -1, 3) == 1           # ... `other` pins the wide kernel
+        assert mil.linear_plan(queue, M, N, K, xb, wb)[0] == 0
+        assert mil.linear_plan(other, M, N, K, xb, wb)[0] == 1
+        assert L.mi_stream_set_modes(other.handle, -1, -1) == 1          # forget: back to the default
+        assert mil.linear_plan(other, M, N, K, xb, wb)[0] == 0
+        assert L.mi_stream_set_modes(other.handle, 5, 0) == 0            # no such gemv mode
+    finally:
+        L.mi_set_gemm_mode(0)
+        L.mi_stream_set_modes(other.handle, -1, -1)
+        mil.nnopt_unregister_weight(wb)

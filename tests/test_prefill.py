@@ -173,6 +173,9 @@ def test_qwen_shaped_prompt_against_single_token_steps_on_device():
     # nine query heads per key/value head: more than a block of the grouped kernel serves, one block per head and row
     ("nine_per_group", dict(hidden=576, inter=1536, n_heads=9, n_kv_heads=1, head_dim=64, n_layers=1, vocab=1024,
                             max_pos=80, rms_eps=1e-5, rope_theta=100000.0), 71),
+    # a head width that is no whole number of wavefronts: the per-head kernels on both sides
+    ("head_dim_80", dict(hidden=640, inter=1024, n_heads=8, n_kv_heads=2, head_dim=80, n_layers=2, vocab=1024,
+                         max_pos=100, rms_eps=1e-6, rope_theta=10000.0), 75),
     # eight heads per group over 1800 positions: 66 KB of scores per block, beyond the 64 KB a kernel gets
     # unasked; checked against the device's own single-token steps (the CPU harness would need 15 s)
     ("long_context", dict(hidden=512, inter=512, n_heads=8, n_kv_heads=1, head_dim=64, n_layers=1, vocab=512,
