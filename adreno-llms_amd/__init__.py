@@ -66,6 +66,7 @@ _SIGNATURES = {
     "mi_decoder_buffer": (_vp, [_vp, _i]),
     "mi_argmax_f16": (_i, [_vp, _vp, _i, _i, _vp]),
     "mi_linear_argmax": (_i, [_vp, _i, _i, _vp, _vp, _vp, _i, _vp]),
+    "mi_linear_argmax_static": (_i, [_vp, _i, _i, _vp, _vp, _vp, _i, _vp]),
     "mi_stream_set_modes": (_i, [_vp, _i, _i]),
     "mi_stream_read_probe": (_i, [_vp, _vp, C.c_size_t, _vp]),
     "mi_linear_plan": (_i, [_vp, _i, _i, _i, _vp, _vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
@@ -304,6 +305,13 @@ def linear_plan(queue, M, N, K, x, W):
     tr, ks = C.c_int(0), C.c_int(1)
     kern = lib().mi_linear_plan(_q(queue), M, N, K, _h(x), _h(W), C.byref(tr), C.byref(ks))
     return kern, tr.value, ks.value
+
+
+def pytorch_linear_argmax_static(queue, N, K, x, W, logits, token_out, num_partials=32):
+    """pytorch_linear_argmax for callers that cannot allocate: the kernels' scratch is an array
+    inside the library (mi_linear_argmax_static); works on any stream."""
+    return bool(lib().mi_linear_argmax_static(_q(queue), N, K, _h(x), _h(W), _h(logits), num_partials,
+                                              _h(token_out)))
 
 
 class DecoderConfig(C.Structure):

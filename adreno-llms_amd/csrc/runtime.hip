@@ -8,6 +8,12 @@
 #include <mutex>
 #include <unordered_map>
 
+// Scratch of mi_linear_argmax_static: lives in the code object, so no call ever allocates it.
+// Every device that runs this library holds its own copy at its own address; the name below is
+// only a host-side handle for hipGetSymbolAddress, never a pointer a kernel can use.
+constexpr size_t kStaticScratchBytes = static_cast<size_t>(mi::kGemvArgmaxMaxSlots) * 8;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace mi {
 namespace {
 
@@ -39,6 +45,11 @@ constexpr size_t kWorkspaceBytes = 16u << 20;
 std::unordered_map<hipStream_t, void*> g_workspace;
 struct StreamModes { int gemv = -1, gemm = -1; };      // -1: the process default
 std::unordered_map<hipStream_t, StreamModes> g_stream_modes;
+
+// Device address of `scratch` (top of this file) per device.
+static_assert(kStaticScratchBytes >= kArgmaxScratchBytes, "the two-launch argmax fits as well");
+constexpr int kMaxDevices = 64;
+void* g_static_scratch[kMaxDevices] = {};     // device address of `scratch` per device, set by mi_init
 
 void* workspace_of(hipStream_t s) {
     std::lock_guard<std::mutex> lk(g_registry_mu);
@@ -132,6 +143,7 @@ bool linear_argmax_in(void* ws, hipStream_t s, int N, int K, const void* x, cons
     c.norm_w = norm_w; c.norm_eps = norm_eps;
     if (!ws || !gemv_takes_argmax(s, c) || (norm_w && !gemv_takes_norm(e.kind, K))) return true;
     static_assert(kGemvArgmaxMaxSlots * 8 <= kWorkspaceBytes, "candidates fit the workspace");
+    static_assert(kGemvArgmaxMaxSlots * 8 <= kStaticScratchBytes, "candidates fit the static scratch");
     c.am_v = static_cast<float*>(ws);
     c.am_i = reinterpret_cast<int*>(c.am_v + kGemvArgmaxMaxSlots);
     c.am_np = num_partials;
@@ -185,6 +197,12 @@ int mi_init(int device) {
         MI_ERROR_FMT("mi_init: device %d is %s; this library holds gfx950 code only", device,
                      prop.gcnArchName);
         return 0;
+    }
+    if (device < kMaxDevices && !g_static_scratch[device]) {
+        // with this device current: the address is the one of this device's copy of the array
+        void* p = nullptr;
+        if (!MI_HIP_OK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) || !p) return 0;
+        g_static_scratch[device] = p;
     }
     g_dev.device = device;
     g_dev.cus = prop.multiProcessorCount;
@@ -390,6 +408,43 @@ int mi_linear_argmax(void* stream, int N, int K, const void* x, const void* W, v
     if (taken) return 1;
     if (!mi_linear(stream, 1, N, K, x, W, logits)) return 0;
     return mi_argmax_f16(stream, logits, N, num_partials, token_out);
+}
+
+int mi_linear_argmax_static(void* stream, int N, int K, const void* x, const void* W, void* logits, int num_partials,
+                            void* token_out) {
+    if (!ensure_init()) return 0;
+    if (N <= 0 || K <= 0 || !x || !W || !logits || !token_out || num_partials <= 0 ||
+        reinterpret_cast<uintptr_t>(token_out) % 4) {
+        MI_ERROR_FMT("mi_linear_argmax_static: bad argument (N=%d K=%d num_partials=%d token_out=%p)", N, K,
+                     num_partials, token_out);
+        return 0;
+    }
+    if (N > MI_LINEAR_ARGMAX_STATIC_MAX_N) {
+        MI_ERROR_FMT("mi_linear_argmax_static: N=%d is beyond the %d rows this entry point takes", N,
+                     MI_LINEAR_ARGMAX_STATIC_MAX_N);
+        return 0;
+    }
+    int device = -1;
+    if (!MI_HIP_OK(hipGetDevice(&device))) return 0;
+    void* ws = device >= 0 && device < kMaxDevices ? g_static_scratch[device] : nullptr;
+    if (!ws) {
+        MI_ERROR_FMT("mi_linear_argmax_static: device %d was not set up by mi_init", device);
+        return 0;
+    }
+    // The candidates of the fused launch (one per wavefront of its grid, every one of them written
+    // by every launch, "none" included) or the 64 partials of the two-launch argmax: nothing in the
+    // scratch has to start at zero, and nothing of an earlier call is read.
+    bool taken = false;
+    if (!linear_argmax_in(ws, as_stream(stream), N, K, x, W, logits, nullptr, 0.0f, num_partials, token_out, nullptr,
+                          nullptr, &taken)) return 0;
+    if (taken) return 1;
+    Entry e;
+    if (!resolve("mi_linear_argmax_static", W, N, K, &e)) return 0;
+    GemvCall c;
+    c.x = x; c.W = W; c.scale = e.scale; c.y = logits;
+    c.M = 1; c.N = N; c.K = K; c.kind = e.kind; c.epi = EPI_STORE;
+    if (!launch_gemv(as_stream(stream), c)) return 0;
+    return launch_argmax_f16(as_stream(stream), logits, N, num_partials, token_out, ws) ? 1 : 0;
 }
 
 // True when [a, a+na) and [b, b+nb) share a byte.

@@ -127,6 +127,20 @@ int mi_argmax_f16(void* stream, const void* logits, int N, int num_partials, voi
 int mi_linear_argmax(void* stream, int N, int K, const void* x, const void* W, void* logits, int num_partials,
                      void* token_out);
 
+/* mi_linear_argmax for callers that cannot allocate or depend on an allocation made for them:
+ * code under HIP graph capture on a stream this library did not create, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, same
+ * logits and token as mi_linear_argmax; the scratch of its kernels (the wavefronts' argmax
+ * candidates, 64 KiB) is an array inside the library's code object instead of a stream's
+ * workspace, so it works on any stream and calls no hipMalloc / hipFree.  Each device holds one
+ * such array, set up by mi_init for that device and kept until the process ends.  All calls on a
+ * device share it: calls that overlap in time on one device (two streams, two threads) race on the
+ * candidates and may return a wrong token; calls on one stream are ordered and safe.
+ * N above MI_LINEAR_ARGMAX_STATIC_MAX_N is refused with an error line. */
+#define MI_LINEAR_ARGMAX_STATIC_MAX_N (1 << 22)
+int mi_linear_argmax_static(void* stream, int N, int K, const void* x, const void* W, void* logits,
+                            int num_partials, void* token_out);
+
 /* One call of mi_linear, for mi_linear_batch. */
 typedef struct mi_linear_call {
     int M, N, K;
