@@ -412,7 +412,11 @@ int mi_linear_argmax(void* stream, int N, int K, const void* x, const void* W, v
 
 int mi_linear_argmax_static(void* stream, int N, int K, const void* x, const void* W, void* logits, int num_partials,
                             void* token_out) {
-    if (!ensure_init()) return 0;
+    // (no lazy set-up here: mi_init allocates the null stream's workspace, and this entry point allocates nothing)
+    if (!g_inited) {
+        MI_ERROR_FMT("mi_linear_argmax_static: mi_init has not run on this process");
+        return 0;
+    }
     if (N <= 0 || K <= 0 || !x || !W || !logits || !token_out || num_partials <= 0 ||
         reinterpret_cast<uintptr_t>(token_out) % 4) {
         MI_ERROR_FMT("mi_linear_argmax_static: bad argument (N=%d K=%d num_partials=%d token_out=%p)", N, K,

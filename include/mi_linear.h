@@ -133,7 +133,9 @@ int mi_linear_argmax(void* stream, int N, int K, const void* x, const void* W, v
  * logits and token as mi_linear_argmax; the scratch of its kernels (the wavefronts' argmax
  * candidates, 64 KiB) is an array inside the library's code object instead of a stream's
  * workspace, so it works on any stream and calls no hipMalloc / hipFree.  Each device holds one
- * such array, set up by mi_init for that device and kept until the process ends.  All calls on a
+ * such array, set up by mi_init for that device (which must have run: this call does no lazy set-up)
+ * and kept until the process ends.  The first launch of a kernel loads its code, so call once before
+ * capturing.  All calls on a
  * device share it: calls that overlap in time on one device (two streams, two threads) race on the
  * candidates and may return a wrong token; calls on one stream are ordered and safe.
  * N above MI_LINEAR_ARGMAX_STATIC_MAX_N is refused with an error line. */
