@@ -61,6 +61,7 @@ _SIGNATURES = {
     "mi_decoder_set_token": (_i, [_vp, _vp, _i]),
     "mi_decoder_step": (_i, [_vp, _vp]),
     "mi_decoder_prefill": (_i, [_vp, _vp, C.POINTER(_i), _i, _i]),
+    "mi_decoder_reserve_prompt": (_i, [_vp, _vp, _i]),
     "mi_decoder_read": (_i, [_vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
     "mi_decoder_logits": (_vp, [_vp]),
     "mi_decoder_buffer": (_vp, [_vp, _i]),
@@ -362,6 +363,10 @@ class Decoder:
         """A prompt at once (Model::forward with seq_len = len(tokens), QW/src/model.cpp:243-376)."""
         arr = (_i * len(tokens))(*[int(t) for t in tokens])
         return bool(lib().mi_decoder_prefill(self.handle, _q(queue), arr, len(tokens), pos0))
+
+    def reserve_prompt(self, queue, max_tokens):
+        """Room (and the stacked projection matrices) for prompts of up to max_tokens tokens, made now."""
+        return bool(lib().mi_decoder_reserve_prompt(self.handle, _q(queue), int(max_tokens)))
 
     def read(self, queue):
         pos, tok = _i(), _i()

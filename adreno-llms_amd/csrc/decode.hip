@@ -1251,6 +1251,70 @@ static void* stack_weights(Decoder* d, hipStream_t s, int n, const void* const* 
     return reg ? w : nullptr;
 }
 
+// Device rows for a prompt of up to M tokens (H, XN, T [M, hidden]; QKV [M, qd + 2 kvd]; QR, ATT
+// [M, qd]; GU [M, 2 inter]; G2 [M, inter]; the token ids).  Grows only; growing waits for the
+// stream (an earlier prompt may still be running in the old rows) and reallocates.
+static bool ensure_prompt_rows(Decoder* d, hipStream_t s, int M) {
+    if (M <= d->prompt_rows) return true;
+    const mi_decoder_config& c = d->c;
+    const size_t qd = static_cast<size_t>(c.n_heads) * c.head_dim, kvd = static_cast<size_t>(c.n_kv_heads) * c.head_dim;
+    const size_t row_halves = 3 * static_cast<size_t>(c.hidden) + 3 * qd + 2 * kvd + 3 * static_cast<size_t>(c.inter);
+    if (d->prompt_mem) {
+        if (!MI_HIP_OK(hipStreamSynchronize(s))) return false;
+        (void)hipFree(d->prompt_mem);
+        d->prompt_mem = nullptr;
+        d->prompt_rows = 0;
+    }
+    // every block starts at a multiple of 16 bytes: the row counts are padded to 8 halves per block
+    const size_t bytes = (row_halves * M + 10 * 8) * 2 + static_cast<size_t>(M) * 4 + 16;
+    if (!MI_HIP_OK(hipMalloc(&d->prompt_mem, bytes))) {
+        d->prompt_mem = nullptr;
+        return false;
+    }
+    d->prompt_rows = M;
+    return true;
+}
+
+// Every layer's q | k | v and gate | up matrices stacked into one registered matrix each, once.
+static bool ensure_stacked(Decoder* d, hipStream_t s) {
+    if (d->stacked_built) return true;
+    const mi_decoder_config& c = d->c;
+    const int Hd = c.hidden, qd = c.n_heads * c.head_dim, kvd = c.n_kv_heads * c.head_dim, I = c.inter;
+    d->wqkv.assign(c.n_layers, nullptr);
+    d->wgu.assign(c.n_layers, nullptr);
+    bool failed = false;
+    for (int l = 0; l < c.n_layers && !failed; ++l) {
+        const void* const W3[3] = {d->wq[l], d->wk[l], d->wv[l]};
+        const int N3[3] = {qd, kvd, kvd};
+        d->wqkv[l] = stack_weights(d, s, 3, W3, N3, Hd, &failed);
+        const void* const W2[2] = {d->wgate[l], d->wup[l]};
+        const int N2[2] = {I, I};
+        if (!failed && I % 4 == 0) d->wgu[l] = stack_weights(d, s, 2, W2, N2, Hd, &failed);
+    }
+    if (failed) {
+        // nothing half-built stays behind: the next prompt starts over, and no registry entry
+        // outlives the memory it names
+        if (!MI_HIP_OK(hipStreamSynchronize(s))) return false;
+        for (void* w : d->wqkv) if (w) mi_unregister_weight(w);
+        for (void* w : d->wgu) if (w) mi_unregister_weight(w);
+        for (void* p : d->stacked_mem) { mi_unregister_weight(p); (void)hipFree(p); }
+        d->wqkv.clear(); d->wgu.clear(); d->stacked_mem.clear();
+        return false;
+    }
+    d->stacked_built = true;
+    return true;
+}
+
+int mi_decoder_reserve_prompt(void* dec, void* stream, int max_tokens) {
+    auto* d = static_cast<Decoder*>(dec);
+    if (!d || max_tokens < 1 || max_tokens > d->c.max_pos) {
+        MI_ERROR_FMT("mi_decoder_reserve_prompt: bad argument (max_tokens=%d, max_pos=%d)", max_tokens, d ? d->c.max_pos : 0);
+        return 0;
+    }
+    auto s = static_cast<hipStream_t>(stream);
+    return ensure_prompt_rows(d, s, max_tokens) && ensure_stacked(d, s) && MI_HIP_OK(hipStreamSynchronize(s)) ? 1 : 0;
+}
+
 int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens, int pos0) {
     auto* d = static_cast<Decoder*>(dec);
     if (!d || !tokens || n_tokens < 1 || pos0 < 0 || static_cast<long>(pos0) + n_tokens > d->c.max_pos) {
@@ -1264,26 +1328,10 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
     const float scale = 1.0f / sqrtf(static_cast<float>(D));
     auto launched = [] { return MI_HIP_OK(hipGetLastError()); };
 
-    // rows of the prompt: H, XN, T [M, hidden]; QKV [M, qd + 2 kvd] (q | k | v of a row side by side
-    // from the stacked projection, or three blocks of their own); QR, ATT [M, qd]; GU [M, 2 inter]
-    // likewise; G2 [M, inter]; tokens
-    const size_t row_halves = 3 * static_cast<size_t>(Hd) + 3 * static_cast<size_t>(qd) + 2 * static_cast<size_t>(kvd) +
-                              3 * static_cast<size_t>(I);
-    if (M > d->prompt_rows) {
-        if (d->prompt_mem) {
-            if (!MI_HIP_OK(hipStreamSynchronize(s))) return 0;      // an earlier prompt may still be running in it
-            (void)hipFree(d->prompt_mem);
-            d->prompt_mem = nullptr;
-            d->prompt_rows = 0;
-        }
-        // every block starts at a multiple of 16 bytes: the row counts are padded to 8 halves per block
-        const size_t bytes = (row_halves * M + 10 * 8) * 2 + static_cast<size_t>(M) * 4 + 16;
-        if (!MI_HIP_OK(hipMalloc(&d->prompt_mem, bytes))) {
-            d->prompt_mem = nullptr;
-            return 0;
-        }
-        d->prompt_rows = M;
-    }
+    // rows of the prompt (allocated here unless mi_decoder_reserve_prompt has made room already):
+    // H, XN, T [M, hidden]; QKV [M, qd + 2 kvd] (q | k | v of a row side by side from the stacked
+    // projection, or three blocks of their own); QR, ATT [M, qd]; GU [M, 2 inter] likewise; G2 [M, inter]; tokens
+    if (!ensure_prompt_rows(d, s, M)) return 0;
     const int cap = d->prompt_rows;
     auto* base = static_cast<uint16_t*>(d->prompt_mem);
     size_t at = 0;
@@ -1296,30 +1344,7 @@ int mi_decoder_prefill(void* dec, void* stream, const int* tokens, int n_tokens,
     uint16_t *GU = carve(2 * static_cast<size_t>(I)), *G2 = carve(I);
     int* tok = reinterpret_cast<int*>(base + at);
 
-    if (!d->stacked_built) {
-        d->wqkv.assign(c.n_layers, nullptr);
-        d->wgu.assign(c.n_layers, nullptr);
-        bool failed = false;
-        for (int l = 0; l < c.n_layers && !failed; ++l) {
-            const void* const W3[3] = {d->wq[l], d->wk[l], d->wv[l]};
-            const int N3[3] = {qd, kvd, kvd};
-            d->wqkv[l] = stack_weights(d, s, 3, W3, N3, Hd, &failed);
-            const void* const W2[2] = {d->wgate[l], d->wup[l]};
-            const int N2[2] = {I, I};
-            if (!failed && I % 4 == 0) d->wgu[l] = stack_weights(d, s, 2, W2, N2, Hd, &failed);
-        }
-        if (failed) {
-            // nothing half-built stays behind: the next prompt starts over, and no registry entry
-            // outlives the memory it names
-            if (!MI_HIP_OK(hipStreamSynchronize(s))) return 0;
-            for (void* w : d->wqkv) if (w) mi_unregister_weight(w);
-            for (void* w : d->wgu) if (w) mi_unregister_weight(w);
-            for (void* p : d->stacked_mem) { mi_unregister_weight(p); (void)hipFree(p); }
-            d->wqkv.clear(); d->wgu.clear(); d->stacked_mem.clear();
-            return 0;
-        }
-        d->stacked_built = true;
-    }
+    if (!ensure_stacked(d, s)) return 0;
     if (!MI_HIP_OK(hipMemcpyAsync(tok, tokens, static_cast<size_t>(M) * 4, hipMemcpyHostToDevice, s))) return 0;
     hipLaunchKernelGGL(embed_rows_kernel, dim3(M), dim3(256), 0, s, static_cast<const uint16_t*>(d->embed), tok, H, Hd, c.vocab);
     if (!launched()) return 0;

@@ -80,6 +80,13 @@ int   mi_decoder_step(void* decoder, void* stream);
  * graph capture.  mi_decoder_buffer(0) afterwards holds the residual
  * stream of the last position; buffers 1 .. 5 are left as they were. */
 int   mi_decoder_prefill(void* decoder, void* stream, const int* tokens, int n_tokens, int pos0);
+/* Does now what the first (or a longer) prompt would otherwise do inside mi_decoder_prefill: makes
+ * the stacked copies of the projection matrices and the activation rows for prompts of up to
+ * max_tokens tokens, and waits for the copies.  After it, mi_decoder_prefill with n_tokens <=
+ * max_tokens allocates nothing, frees nothing and waits for nothing (it still copies the token ids
+ * from host memory, so it stays out of graph capture).  No counterpart in the reference, whose
+ * layers allocate their activation buffers on first use (QW/src/layers/mlp.cpp:228-232). */
+int   mi_decoder_reserve_prompt(void* decoder, void* stream, int max_tokens);
 
 /* Reads the device state back (synchronises the stream). */
 int   mi_decoder_read(void* decoder, void* stream, int* pos, int* token);

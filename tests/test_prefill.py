@@ -95,6 +95,42 @@ def test_prompt_in_two_parts_and_after_steps():
 
 
 @pytest.mark.gpu
+def test_reserved_prompt_room_means_no_allocation_in_prefill():
+    """After mi_decoder_reserve_prompt the prompts that fit allocate nothing (the device's free memory
+    does not move across them) and give the results of a decoder that made its room on the way."""
+    import ctypes
+    assert mil.lib().mi_init(0) == 1
+    hip = ctypes.CDLL("libamdhip64.so")
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    mil.lib().mi_set_gemm_mode(1)
+    try:
+        queue = mil.Queue()
+        m = Model(SMOL, seed=6)
+        prompt = _prompt(40, SMOL["vocab"], 11)
+        want, _, logits = _oracle(m, prompt, 1)
+        gd = GpuDecoder(m, queue)
+        assert not gd.dec.reserve_prompt(queue, 0) and not gd.dec.reserve_prompt(queue, SMOL["max_pos"] + 1)
+        assert gd.dec.reserve_prompt(queue, 40)
+        before = free_bytes()
+        assert gd.dec.prefill(queue, prompt[:17]) and gd.dec.prefill(queue, prompt[17:], 17)
+        assert gd.dec.prefill(queue, prompt)
+        queue.finish()
+        assert free_bytes() == before
+        assert gd.dec.read(queue) == (40, want[0])
+        assert np.array_equal(gd.logits(), logits)
+        assert gd.dec.reserve_prompt(queue, 12)            # less than there is: nothing to do
+        assert free_bytes() == before
+        gd.close()
+    finally:
+        mil.lib().mi_set_gemm_mode(0)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("name,cfg,n_prompt", [("smol", SMOL, 40), ("tiny", TINY, 33), ("smol-f16", SMOL, 40),
                                                ("smol-q4", SMOL, 40)])
 def test_prompt_on_the_matrix_cores_within_tolerance(name, cfg, n_prompt):
