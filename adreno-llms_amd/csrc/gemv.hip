@@ -921,6 +921,8 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
         MI_FIXED(896, true)
         MI_FIXED(1024, true)
         MI_FIXED(1536, true)
+        MI_FIXED(2560, false)         // LFM2's K values beside 1024: the reference ships kernels for exactly these
+        MI_FIXED(4608, false)         // (LF/kernels/gemv_m1_int8.cl:155-255, gemv_m1_q4.cl:128-281)
         MI_FIXED(4864, false)
         default: {
             const size_t lds = static_cast<size_t>(K) * 2;
