@@ -690,8 +690,10 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict_
         const int row = (rb - sg.first) * RPW + r;
         const bool valid = row < sg.N;
         const int rowc = valid ? row : sg.N - 1;
-        const uint8_t* wrow = sg.W + static_cast<size_t>(rowc) * rowb + koff / T::EPV * T::BPV;
-        const uint16_t* srow = sg.sc + static_cast<size_t>(rowc) * (K / 32) + (g * VL) / 4;
+        const uint8_t* row0 = sg.W + static_cast<size_t>(rowc) * rowb;
+        const uint8_t* wrow = row0 + koff / T::EPV * T::BPV;
+        [[maybe_unused]] const uint16_t* srow0 = sg.sc + static_cast<size_t>(rowc) * (K / 32);
+        [[maybe_unused]] const uint16_t* srow = srow0 + (g * VL) / 4;
         float acc[VL];
         #pragma unroll
         for (int v = 0; v < VL; ++v) acc[v] = 0.0f;
@@ -706,10 +708,11 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict_
             for (int u = 0; u < kChunk; ++u) {
                 const int j = j0 + u;
                 if (j >= nit) break;                                  // (uniform: nothing is requested past the row's end)
-                // lanes idle in a partial last iteration re-read the start of their row (the value is never used)
+                // lanes idle in a partial last iteration re-read the first bytes of the row, which every
+                // row has (the value is never used; their own offset may lie past the end of the matrix)
                 const bool active = j * EIT + koff < K;
-                load_dwords<WD, true>(wbuf[b][u], wrow + (active ? static_cast<size_t>(j) * ITB : 0));
-                if constexpr (KIND == WK_Q4) sbuf[b][u] = srow[active ? j * 16 : 0];
+                load_dwords<WD, true>(wbuf[b][u], active ? wrow + static_cast<size_t>(j) * ITB : row0);
+                if constexpr (KIND == WK_Q4) sbuf[b][u] = active ? srow[j * 16] : srow0[0];
             }
         };
         auto multiply_chunk = [&](int b, int j0) {
@@ -769,6 +772,7 @@ __global__ __launch_bounds__(kBlock) void gate_up_silu_any_k(const uint16_t* __r
     constexpr int XD = VL * T::EPV / 2;
     constexpr int WD = VL * T::BPV / 4;
     constexpr int ITB = kWave * T::BPV;
+    constexpr int kChunk = 2;                           // K-iterations of each matrix per register buffer (4 and 8 measured no better)
     extern __shared__ uint32_t xs[];
     for (int i = threadIdx.x; i < K / 2; i += kBlock) xs[i] = reinterpret_cast<const uint32_t*>(x)[i];
     __syncthreads();
@@ -786,25 +790,52 @@ __global__ __launch_bounds__(kBlock) void gate_up_silu_any_k(const uint16_t* __r
         const int row = rb * RPW + r;
         const bool valid = row < N;
         const int rowc = valid ? row : N - 1;
-        const size_t off = static_cast<size_t>(rowc) * rowb + koff / T::EPV * T::BPV;
+        const size_t off0 = static_cast<size_t>(rowc) * rowb;
+        const size_t off = off0 + koff / T::EPV * T::BPV;
         float ag[VL], au[VL];
         #pragma unroll
         for (int v = 0; v < VL; ++v) { ag[v] = 0.0f; au[v] = 0.0f; }
-        #pragma unroll 2
-        for (int j = 0; j < nit; ++j) {
-            const int k = j * EIT + koff;
-            if (k < K) {
-                uint32_t wg[WD], wu[WD], xr[XD];
-                load_dwords<WD, true>(wg, Wg + off + static_cast<size_t>(j) * ITB);
-                load_dwords<WD, true>(wu, Wu + off + static_cast<size_t>(j) * ITB);
-                #pragma unroll
-                for (int i = 0; i < XD; ++i) xr[i] = xs[k / 2 + i];
-                #pragma unroll
-                for (int v = 0; v < VL; ++v) {
-                    ag[v] = vlane_step<KIND>(ag[v], &wg[v * T::BPV / 4], &xr[v * T::EPV / 2], 0.0f, cst);
-                    au[v] = vlane_step<KIND>(au[v], &wu[v * T::BPV / 4], &xr[v * T::EPV / 2], 0.0f, cst);
+        // two register buffers of kChunk K-iterations of both matrices, as in gemv_any_k: one on its
+        // way while the other is multiplied; the additions keep the loop's order
+        uint32_t gbuf[2][kChunk][WD], ubuf[2][kChunk][WD];
+        auto fetch_chunk = [&](int b, int j0) {
+            #pragma unroll
+            for (int u = 0; u < kChunk; ++u) {
+                const int j = j0 + u;
+                if (j >= nit) break;
+                // lanes idle in a partial last iteration re-read the first bytes of the row, which every
+                // row has (the value is never used; their own offset may lie past the end of the matrix)
+                const size_t at = j * EIT + koff < K ? off + static_cast<size_t>(j) * ITB : off0;
+                load_dwords<WD, true>(gbuf[b][u], Wg + at);
+                load_dwords<WD, true>(ubuf[b][u], Wu + at);
+            }
+        };
+        auto multiply_chunk = [&](int b, int j0) {
+            #pragma unroll
+            for (int u = 0; u < kChunk; ++u) {
+                const int j = j0 + u, k = j * EIT + koff;
+                if (j < nit && k < K) {
+                    uint32_t xr[XD];
+                    #pragma unroll
+                    for (int i = 0; i < XD; ++i) xr[i] = xs[k / 2 + i];
+                    #pragma unroll
+                    for (int v = 0; v < VL; ++v) {
+                        ag[v] = vlane_step<KIND>(ag[v], &gbuf[b][u][v * T::BPV / 4], &xr[v * T::EPV / 2], 0.0f, cst);
+                        au[v] = vlane_step<KIND>(au[v], &ubuf[b][u][v * T::BPV / 4], &xr[v * T::EPV / 2], 0.0f, cst);
+                    }
                 }
             }
+        };
+        fetch_chunk(0, 0);
+        for (int j0 = 0;;) {
+            if (j0 + kChunk < nit) fetch_chunk(1, j0 + kChunk);
+            multiply_chunk(0, j0);
+            j0 += kChunk;
+            if (j0 >= nit) break;
+            if (j0 + kChunk < nit) fetch_chunk(0, j0 + kChunk);
+            multiply_chunk(1, j0);
+            j0 += kChunk;
+            if (j0 >= nit) break;
         }
         float gs = reduce_row<VL>(ag);
         float us = reduce_row<VL>(au);
