@@ -821,6 +821,318 @@ bool launch_any(int tm, hipStream_t s, int M, int N, int K, const void* x, const
 
 }  // namespace wide
 
+// ---- a few rows of x (M <= 64): the weights stream once, as in the GEMV ------------------------
+//
+// With up to 64 rows of x the contraction is bound by the weights' bytes, like the GEMV, not by
+// the matrix cores, and the tiles above leave most of the chip idle (19 tiles at N = 4864).  Here a
+// wavefront takes a strip of 16 rows of W and streams it through v_mfma_f32_16x16x32_f16 against
+// the 16 MT rows of x:
+//   A = W strip: lane l supplies row l % 16, 8 values of K starting at 16 (l / 16) + 8 s of the
+//       iteration's 64 (s = 0, 1: the two MFMAs of an iteration), i.e. one 16-byte load of int8
+//       weights per lane and iteration, 64 contiguous bytes per row;
+//   B = x^T: lane l supplies row l % 16 of the x tile at the same 16 values of K, 32 contiguous
+//       bytes (x is small and comes from the caches);
+//   D[i][j] (lane l: i = 4 (l / 16) + r, j = l % 16) = out[row j of the x tile][row i of the strip]:
+//       four consecutive output columns per lane.
+// K is cut into ks slices over the wavefronts of a block where N alone gives too few strips to
+// fill the chip; their sums meet in LDS and are added in slice order.  Iterations go through two
+// register buffers, one in flight while the other is multiplied.
+namespace skinny {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+constexpr int kMaxM = 64;
+constexpr int kWaves = 8;                // wavefronts per block
+
+// SW strips of W per wavefront: the fragments of x a lane holds are multiplied with SW strips.
+// XL: the block first copies its rows of x into LDS (rows padded by 16 bytes, which spreads the 16
+// rows a 16-byte read touches over all banks) and every wavefront reads its fragments from there;
+// blocks then live long and walk over the strips.  Without XL (x too large for LDS) the fragments
+// come from the caches with the weights, 2 MT / SW bytes per byte of W, and the L1's few requests
+// in flight bound the rate: that form only pays for a few rows of x at a long K.
+template <int KIND, int MT, int SW, bool XL>
+__global__ __launch_bounds__(64 * kWaves) void gemm_skinny(const uint16_t* __restrict__ X,
+                                                           const uint8_t* __restrict__ W,
+                                                           const uint16_t* __restrict__ scale,
+                                                           uint16_t* __restrict__ out, int M, int N, int K, int ks,
+                                                           int logical_blocks) {
+    constexpr bool F16 = KIND == WK_F16;
+    constexpr int WV = F16 ? 2 : 1;                       // 16-byte loads of W per lane, strip and iteration
+    constexpr int kWB = F16 ? 2 : 1;                      // bytes per weight
+    constexpr int kPerIt = 4 * SW * WV + (XL ? 0 : 8 * MT);   // registers one iteration's operands take in a buffer
+    constexpr int kChunk = 64 / kPerIt < 1 ? 1 : 64 / kPerIt > 8 ? 8 : 64 / kPerIt;   // iterations per register buffer
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint32_t xrow = XL ? static_cast<uint32_t>(K) * 2u + 16u : 0u;              // bytes per row of x in LDS
+    float* red = reinterpret_cast<float*>(lds + 16u * MT * xrow);                     // [kWaves][MT][4][64]
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i = lane & 15, c = lane >> 4;
+    const int slice = wave % ks;
+    const int nit = K / 64;
+    const int it0 = nit * slice / ks, it1 = nit * (slice + 1) / ks;
+
+    if constexpr (XL) {
+        const int per_row = K / 8;                       // 16-byte pieces per row
+        for (int idx = threadIdx.x; idx < 16 * MT * per_row; idx += 64 * kWaves) {
+            const int row = idx / per_row, piece = idx - row * per_row;
+            const int m = row < M ? row : M - 1;         // rows past M are read as the last row (and never stored)
+            *reinterpret_cast<u32x4*>(lds + row * xrow + piece * 16) =
+                *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint8_t*>(X) + static_cast<size_t>(m) * K * 2 + piece * 16);
+        }
+        __syncthreads();
+    }
+    const uint8_t* xp[MT];                               // without XL: this lane's rows of x in memory
+    #pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = 16 * t + i < M ? 16 * t + i : M - 1;
+        xp[t] = reinterpret_cast<const uint8_t*>(X) + static_cast<size_t>(m) * K * 2 + c * 32;
+    }
+    const uint32_t xl = (16u * 0 + i) * xrow + c * 32u;  // with XL: this lane's row of the first x tile in LDS
+    const bool cols4 = (N % 4) == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0;
+
+    for (int lb = blockIdx.x; lb < logical_blocks; lb += gridDim.x) {     // (the same trips for the whole block)
+        const int group = lb * (kWaves / ks) + wave / ks;                 // group: SW consecutive strips
+        const uint8_t* wp[SW];
+        #pragma unroll
+        for (int q = 0; q < SW; ++q) {
+            const int row = 16 * (group * SW + q) + i;                    // rows past N are read as the last row
+            wp[q] = W + static_cast<size_t>(row < N ? row : N - 1) * K * kWB + c * 16 * WV;
+        }
+        floatx4 acc[SW][MT];
+        #pragma unroll
+        for (int q = 0; q < SW; ++q)
+            #pragma unroll
+            for (int t = 0; t < MT; ++t) acc[q][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+
+        u32x4 wb[2][kChunk][SW][WV];
+        [[maybe_unused]] u32x4 xb[2][XL ? 1 : kChunk][XL ? 1 : MT][2];
+        // `full`: kChunk iterations whatever the slice's end (the caller knows they exist); the number
+        // of requests is then a constant, and only then can the wait before a buffer is multiplied
+        // leave the other buffer's requests in flight
+        auto fetch = [&](auto fullc, int b, int j0) {
+            #pragma unroll
+            for (int u = 0; u < kChunk; ++u) {
+                const int it = j0 + u;
+                if constexpr (!decltype(fullc)::value) {
+                    if (it >= it1) break;
+                }
+                if constexpr (!XL) {
+                    #pragma unroll
+                    for (int t = 0; t < MT; ++t)
+                        #pragma unroll
+                        for (int e = 0; e < 2; ++e)
+                            xb[b][u][t][e] = reinterpret_cast<const u32x4*>(xp[t] + static_cast<size_t>(it) * 128)[e];
+                }
+                #pragma unroll
+                for (int q = 0; q < SW; ++q)
+                    #pragma unroll
+                    for (int v = 0; v < WV; ++v)
+                        wb[b][u][q][v] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp[q] + static_cast<size_t>(it) * 64 * kWB) + v);
+            }
+        };
+        auto multiply = [&](int b, int j0) {
+            #pragma unroll
+            for (int u = 0; u < kChunk; ++u) {
+                if (j0 + u < it1) {
+                    half8 xf[MT][2];
+                    #pragma unroll
+                    for (int t = 0; t < MT; ++t)
+                        #pragma unroll
+                        for (int e = 0; e < 2; ++e) {
+                            if constexpr (XL)
+                                xf[t][e] = *reinterpret_cast<const half8*>(lds + xl + 16u * t * xrow + (j0 + u) * 128 + 16 * e);
+                            else
+                                xf[t][e] = __builtin_bit_cast(half8, xb[b][u][t][e]);
+                        }
+                    #pragma unroll
+                    for (int q = 0; q < SW; ++q) {
+                        half8 a[2];
+                        if constexpr (F16) {
+                            a[0] = __builtin_bit_cast(half8, wb[b][u][q][0]);
+                            a[1] = __builtin_bit_cast(half8, wb[b][u][q][1]);
+                        } else {
+                            uint32_t h[8];
+                            i8x4_to_h4(wb[b][u][q][0].x, h[0], h[1]);
+                            i8x4_to_h4(wb[b][u][q][0].y, h[2], h[3]);
+                            i8x4_to_h4(wb[b][u][q][0].z, h[4], h[5]);
+                            i8x4_to_h4(wb[b][u][q][0].w, h[6], h[7]);
+                            a[0] = __builtin_bit_cast(half8, u32x4{h[0], h[1], h[2], h[3]});
+                            a[1] = __builtin_bit_cast(half8, u32x4{h[4], h[5], h[6], h[7]});
+                        }
+                        #pragma unroll
+                        for (int t = 0; t < MT; ++t)
+                            #pragma unroll
+                            for (int e = 0; e < 2; ++e)
+                                acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[e], xf[t][e], acc[q][t], 0, 0, 0);
+                    }
+                }
+            }
+        };
+        // buffers 0 and 1 in turn while two more whole chunks lie ahead; then what is left (one
+        // buffer that may be on its way already, and at most one more chunk)
+        int j0 = it0, cur = 0;
+        if (it1 - j0 >= 2 * kChunk) {
+            fetch(std::true_type{}, 0, j0);
+            while (true) {
+                fetch(std::true_type{}, 1, j0 + kChunk);
+                multiply(0, j0);
+                j0 += kChunk;
+                if (it1 - j0 < 2 * kChunk) { cur = 1; break; }
+                fetch(std::true_type{}, 0, j0 + kChunk);
+                multiply(1, j0);
+                j0 += kChunk;
+                if (it1 - j0 < 2 * kChunk) { cur = 0; break; }
+            }
+        } else {
+            fetch(std::false_type{}, 0, j0);
+        }
+        if (cur == 0) {
+            fetch(std::false_type{}, 1, j0 + kChunk);
+            multiply(0, j0);
+            multiply(1, j0 + kChunk);
+        } else {
+            fetch(std::false_type{}, 0, j0 + kChunk);
+            multiply(1, j0);
+            multiply(0, j0 + kChunk);
+        }
+
+        if (ks > 1) {                                    // (the same for every wavefront of the grid)
+            #pragma unroll
+            for (int q = 0; q < SW; ++q) {               // one strip at a time through the same 4 MT KB per wavefront
+                __syncthreads();                         // the last round's sums have been read
+                if (slice > 0) {
+                    #pragma unroll
+                    for (int t = 0; t < MT; ++t)
+                        #pragma unroll
+                        for (int r = 0; r < 4; ++r) red[((wave * MT + t) * 4 + r) * 64 + lane] = acc[q][t][r];
+                }
+                __syncthreads();
+                if (slice == 0) {
+                    for (int z = 1; z < ks; ++z) {       // slice 0 + slice 1 + ..., in this order
+                        #pragma unroll
+                        for (int t = 0; t < MT; ++t)
+                            #pragma unroll
+                            for (int r = 0; r < 4; ++r) acc[q][t][r] += red[(((wave + z) * MT + t) * 4 + r) * 64 + lane];
+                    }
+                }
+            }
+            if (slice > 0) continue;
+        }
+
+        #pragma unroll
+        for (int q = 0; q < SW; ++q) {
+            const int nq = 16 * (group * SW + q) + 4 * c;    // first of this lane's 4 output columns
+            if (nq >= N) continue;
+            float s4[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+            if constexpr (KIND == WK_I8) {
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) s4[r] = __half2float(__ushort_as_half(scale[nq + r < N ? nq + r : N - 1]));
+            }
+            #pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const int m = 16 * t + i;
+                if (m >= M) continue;
+                const uint32_t lo = wide::pack_half2(acc[q][t][0] * s4[0], acc[q][t][1] * s4[1]);
+                const uint32_t hi = wide::pack_half2(acc[q][t][2] * s4[2], acc[q][t][3] * s4[3]);
+                uint16_t* dst = out + static_cast<size_t>(m) * N + nq;
+                if (cols4 && nq + 3 < N) {
+                    *reinterpret_cast<uint2*>(dst) = uint2{lo, hi};
+                } else {
+                    #pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (nq + r < N) dst[r] = static_cast<uint16_t>((r / 2 ? hi : lo) >> (16 * (r % 2)));
+                }
+            }
+        }
+    }
+}
+
+constexpr size_t kLdsLimit = 160 * 1024;
+// bytes of LDS a block takes: the rows of x (XL) and the buffer in which K-slices meet
+inline size_t lds_bytes(int mt, int K, bool xl, int ks) {
+    return (xl ? static_cast<size_t>(16) * mt * (2 * static_cast<size_t>(K) + 16) : 0) +
+           (ks > 1 ? static_cast<size_t>(kWaves) * mt * 4 * 64 * 4 : 0);
+}
+
+struct Shape { int ks; bool xl; };
+// Slices of K per strip (1, 2, 4, 8: the fewest that give the chip four wavefronts per CU; measured
+// at 4864 x 896: 4 slices 4.5 us, 8 slices 6.7 us), x in LDS where it fits.  One strip per wavefront:
+// two and four (the kernel's SW) were measured slower at every shape tried (fewer wavefronts; the
+// reads of x they save are not the bound).
+inline Shape pick_shape(int M, int N, int K, int cus) {
+    const int mt = (M + 15) / 16;
+    const long strips = (N + 15) / 16;
+    Shape sh{1, false};
+    while (sh.ks < kWaves && strips * sh.ks < 4L * cus && K / 64 >= 2 * sh.ks) sh.ks *= 2;
+    sh.xl = lds_bytes(mt, K, true, sh.ks) <= kLdsLimit;
+    return sh;
+}
+
+// Where the streaming kernel is the library's own choice (measured against the tiles above, int8,
+// warm weights): up to 32 rows of x with x in LDS (4864 x 896: 4.5 / 5.6 us at 16 / 32 rows against
+// 6.6 / 6.7 us; 48 rows tie, 64 rows lose, 7.6 against 6.8 us), up to 16 rows when x has to come
+// from the caches (896 x 4864: 10.0 against 12.1 us), and no more strips than stay resident at
+// once: an lm_head of 151 936 rows streams at 4.0 TB/s here (a wavefront loads a strip, waits,
+// multiplies) against 4.8 TB/s in the wide kernel.
+inline bool preferred(int M, int N, int K, int cus) {
+    const Shape sh = pick_shape(M, N, K, cus);
+    return M <= (sh.xl ? 32 : 16) && (N + 15) / 16 <= 16L * cus;
+}
+
+// Estimated time (us), fitted to the same measurements.
+inline double estimate_us(int kind, int M, int N, int K, int cus) {
+    const Shape sh = pick_shape(M, N, K, cus);
+    const double w_bytes = static_cast<double>(N) * K * (kind == WK_F16 ? 2.0 : 1.0);
+    return sh.xl ? 3.75 + 0.035 * M + w_bytes / 8.0e6 : 5.5 + 0.22 * M + w_bytes / 8.0e6;
+}
+
+template <int KIND, int MT, int SW, bool XL>
+bool launch_one(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, int ks) {
+    const long groups = ((N + 15) / 16 + SW - 1) / SW, per_block = kWaves / ks;
+    const long logical = (groups + per_block - 1) / per_block;
+    const size_t lds = lds_bytes(MT, K, XL, ks);
+    auto* kern = gemm_skinny<KIND, MT, SW, XL>;
+    if (lds > 65536 &&
+        !MI_ONCE_OK(MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsLimit)))))
+        return false;
+    // with x in LDS a block is worth keeping: as many as fit a CU at once (by LDS; at most 4), each walking over the strips
+    long grid = logical;
+    if (XL) {
+        const long per_cu = lds == 0 ? 4 : static_cast<long>(kLdsLimit / lds) < 4 ? static_cast<long>(kLdsLimit / lds) : 4;
+        const long resident = static_cast<long>(device_info().cus) * (per_cu < 1 ? 1 : per_cu);
+        if (grid > resident) grid = resident;
+    }
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(64 * kWaves), lds, s, static_cast<const uint16_t*>(x),
+                       static_cast<const uint8_t*>(W), static_cast<const uint16_t*>(scale), static_cast<uint16_t*>(out),
+                       M, N, K, ks, static_cast<int>(logical));
+    return MI_HIP_OK(hipGetLastError());
+}
+
+template <int KIND, int MT>
+bool launch_mt(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, Shape sh) {
+    return sh.xl ? launch_one<KIND, MT, 1, true>(s, M, N, K, x, W, scale, out, sh.ks)
+                 : launch_one<KIND, MT, 1, false>(s, M, N, K, x, W, scale, out, sh.ks);
+}
+
+template <int KIND>
+bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, Shape sh) {
+    if (M < 1 || M > kMaxM || !(sh.ks == 1 || sh.ks == 2 || sh.ks == 4 || sh.ks == 8) ||
+        lds_bytes((M + 15) / 16, K, sh.xl, sh.ks) > kLdsLimit) {
+        MI_ERROR_FMT("gemm: the streaming kernel takes up to %d rows of x, 1, 2, 4 or 8 slices of K and %zu bytes of LDS "
+                     "(M=%d K=%d, %d slices, x in LDS %d)", kMaxM, kLdsLimit, M, K, sh.ks, static_cast<int>(sh.xl));
+        return false;
+    }
+    switch ((M + 15) / 16) {
+        case 1: return launch_mt<KIND, 1>(s, M, N, K, x, W, scale, out, sh);
+        case 2: return launch_mt<KIND, 2>(s, M, N, K, x, W, scale, out, sh);
+        case 3: return launch_mt<KIND, 3>(s, M, N, K, x, W, scale, out, sh);
+        default: return launch_mt<KIND, 4>(s, M, N, K, x, W, scale, out, sh);
+    }
+}
+
+}  // namespace skinny
+
 template <int BM, int BN, int WM, int WN>
 bool launch_tile(hipStream_t s, WeightKind kind, int M, int N, int K, const void* x, const void* W,
                  const void* scale, void* out) {
@@ -889,6 +1201,8 @@ double gemm_estimate_us(WeightKind kind, int M, int N, int K, size_t workspace_b
     if (wide_reaches(kind, M, N, K))
         wide::pick_shape(kind, terms, M, N, K, device_info().cus, workspace_bytes, &tm, &splits, &wide_us);
     if (kind == WK_Q4) return wide_us;
+    if (M <= skinny::kMaxM && skinny::preferred(M, N, K, device_info().cus))
+        return skinny::estimate_us(kind, M, N, K, device_info().cus);
     const double tiled_us = tiled_estimate_us(M, N, K);
     return wide_us < tiled_us ? wide_us : tiled_us;
 }
@@ -912,7 +1226,13 @@ GemmPlan plan_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, size_t w
         p.kernel = 1; p.tile_rows = 32 * tm; p.k_slices = splits;
         return p;
     }
-    // int8 and fp16: the wide kernel where its estimated time beats that of the 64 x 64 tiles
+    // int8 and fp16, a few rows of x: the streaming kernel (mode 5 asks for it by name, up to 64 rows)
+    if (M <= skinny::kMaxM && (mode == 5 || (mode == 0 && skinny::preferred(M, N, K, cus)))) {
+        p.kernel = 4; p.tile_rows = 16 * ((M + 15) / 16); p.k_slices = skinny::pick_shape(M, N, K, cus).ks;
+        return p;
+    }
+    if (mode == 5) return p;
+    // the wide kernel where its estimated time beats that of the 64 x 64 tiles
     if (wide_fits && (mode == 0 || mode == 3 || (mode >= 11 && mode <= 15))) {
         double wide_us = 0.0;
         // modes 3 and 11..15 pin the plain kernel; slices of K are the library's own choice (mode 0)
@@ -951,6 +1271,9 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
             if (kind == WK_F16) return wide::launch_any<WK_F16, 1>(tm, s, M, N, K, x, W, scale, out, partial, ws_bytes, p.k_slices);
             return wide::launch_any<WK_I8, 1>(tm, s, M, N, K, x, W, scale, out, partial, ws_bytes, p.k_slices);
         }
+        case 4:
+            return kind == WK_F16 ? skinny::launch<WK_F16>(s, M, N, K, x, W, scale, out, skinny::pick_shape(M, N, K, device_info().cus))
+                                  : skinny::launch<WK_I8>(s, M, N, K, x, W, scale, out, skinny::pick_shape(M, N, K, device_info().cus));
         case 2: return launch_tile<64, 64, 32, 32>(s, kind, M, N, K, x, W, scale, out);
         case 3: return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);
         default:

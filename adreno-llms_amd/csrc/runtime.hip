@@ -339,14 +339,15 @@ int mi_stream_set_modes(void* stream, int gemv_mode, int gemm_mode) {
 // M > 1: a real contraction goes to the MFMA GEMM.  Every batch in mode 1, and shapes the GEMM
 // does not take, run the GEMV once per row of x, as the reference's quantised prefill does; so
 // do batches below 16 rows while that is estimated to be faster (each GEMV row streams W again:
-// about bytes / 6.6 TB/s, or 1 us when W stays in the caches).
+// about 0.25 us + bytes / 6.6 TB/s per row; measured int8, warm: 1536 x 576 2.95 us for two rows,
+// 4864 x 896 3.8 / 5.0 us and 896 x 4864 3.85 / 6.15 us for two / four).
 static bool takes_gemm(hipStream_t s, const Entry& e, int M, int N, int K, const void* x, const void* W) {
     const int mode = gemm_mode(s);
     if (M < 2 || mode == 1 || !gemm_supported(e.kind, M, N, K, x, W, e.scale)) return false;
     if (M >= 16 || mode != 0) return true;
     const double w_bytes = static_cast<double>(N) * K * (e.kind == WK_F16 ? 2.0 : e.kind == WK_I8 ? 1.0 : 0.5625);
-    const double row_us = w_bytes / 6.6e6 > 1.0 ? w_bytes / 6.6e6 : 1.0;
-    return gemm_estimate_us(e.kind, M, N, K, workspace_of(s) ? kWorkspaceBytes : 0) < 2.5 + M * row_us;
+    const double row_us = 0.25 + w_bytes / 6.6e6;
+    return gemm_estimate_us(e.kind, M, N, K, workspace_of(s) ? kWorkspaceBytes : 0) < 2.4 + M * row_us;
 }
 
 int mi_linear(void* stream, int M, int N, int K, const void* x, const void* W, void* out) {

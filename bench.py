@@ -409,7 +409,10 @@ def main():
                 ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 1, 9) / 20
                 flop = 2.0 * M * N * K
                 nbytes = 2 * M * K + N * K + 2 * N + 2 * M * N
+                kern, rows, slices = mil.linear_plan(queue, M, N, K, xb, wb)
                 detail[f"c5_int8_gemm_M{M}_N{N}_K{K}"] = {
+                    "kernel": {1: "wide", 2: "tile64", 3: "tile128", 4: "streaming"}.get(kern, str(kern)),
+                    "rows_of_x_per_block": rows, "k_slices": slices,
                     "us": round(ms * 1e3, 2), "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 1),
                     "frac_mfma_fp16_peak": round(flop / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4),
                     "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),

@@ -167,13 +167,15 @@ int   mi_graph_destroy(void* graph);
 
 /* Selects how M > 1 is computed: 0 (default) = MFMA GEMM with fused dequant for M >= 16, and
  * for 2 <= M < 16 where it is estimated to beat M rows of GEMV (each row streams W again; e.g. an
- * lm_head from M = 2, an MLP projection from M = 4 to 10); K not a multiple of 64 or operands
+ * lm_head from M = 2, an MLP projection from M = 3 to 6); K not a multiple of 64 or operands
  * not 16-byte aligned always take the batched GEMV; 1 = always the batched GEMV, whose rows
  * are bit-identical to M = 1 calls (the reference's prefill loop, LF/src/model.cpp:243-250);
  * 2, 3 and 11..15 = as 0 with the kernel choice pinned (tests and tuning: results stay within
  * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel (int8 and fp16
  * weights; fails for Q4), 3 = the wide kernel, 10 + t (t = 1..5) = the wide kernel with 32 t
- * rows of x per block.
+ * rows of x per block, 5 = the streaming kernel for up to 64 rows of x (int8 and fp16 weights, which
+ * take it by themselves in mode 0 up to 32 rows where it is the faster one; fails for more than 64
+ * rows; Q4 weights take the wide kernel).
  * Q4 weights: a weight q * scale (4 and 11 significant bits) is not an fp16 number in general.
  * Every mode but 4 feeds it to the matrix cores exactly, as two fp16 terms q * hi + q * lo with
  * scale = hi + lo, and stays within one fp16 step of the batched GEMV.  Mode 4 = as 0, but each
@@ -199,8 +201,10 @@ int mi_stream_set_modes(void* stream, int gemv_mode, int gemm_mode);
 /* What mi_linear(stream, M, N, K, x, W, out) would run, without running it: 0 = GEMV (once per
  * row of x), 1 = the wide MFMA kernel with *tile_rows rows of x per block and K cut into
  * *k_slices slices (more than one slice: fp32 partial sums in the stream's workspace and a
- * reduction launch), 2 / 3 = the 64 x 64 / 128 x 128 tile kernel, -1 = bad arguments.  For
- * tests and tuning; tile_rows and k_slices may be NULL. */
+ * reduction launch), 2 / 3 = the 64 x 64 / 128 x 128 tile kernel, 4 = the streaming kernel for up
+ * to 64 rows of x (*tile_rows = M rounded up to 16, *k_slices = wavefronts of a block that share
+ * one strip of 16 rows of W), -1 = bad arguments.  For tests and tuning; tile_rows and k_slices
+ * may be NULL. */
 int mi_linear_plan(void* stream, int M, int N, int K, const void* x, const void* W, int* tile_rows, int* k_slices);
 
 /* Streaming-read probe: reads `bytes` (a multiple of 16 is read; src 16-byte aligned) from src

@@ -36,8 +36,8 @@ def _ulp_apart(a_u16, b_u16):
 def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0, plan=None):
     """tile is the mi_set_gemm_mode value: 0 = the library's own choice, 1 = rows of GEMV,
     2 = the 64 x 64 MFMA kernel, 3 = the wide kernel with its own choice of rows of x per
-    block, 4 = Q4 weights rounded to fp16 once, 11..15 = the wide kernel with 32, 64, .. 160 rows
-    of x per block.  plan: a list that receives (kernel, rows of x per block, slices of K) of the call."""
+    block, 4 = Q4 weights rounded to fp16 once, 5 = the streaming kernel for up to 64 rows of x,
+    11..15 = the wide kernel with 32, 64, .. 160 rows of x per block.  plan: a list that receives (kernel, rows of x per block, slices of K) of the call."""
     xb, wb = mil.Buffer.from_host(X), mil.Buffer.from_host(W_host)
     sb = mil.Buffer.from_host(scale_host) if scale_host is not None else None
     if kind == "i8":
@@ -151,6 +151,105 @@ def test_gemm_repeats_identically(queue, tile):
         mil.lib().mi_set_gemm_mode(0)
     first = outs[0].read(np.uint16, (M, N))
     assert_tolerance(first.view(np.float16), want.view(np.float16))
+    for i, ob in enumerate(outs[1:]):
+        assert np.array_equal(ob.read(np.uint16, (M, N)), first), f"launch {i + 1} differs from launch 0"
+    mil.nnopt_unregister_weight(wb)
+
+
+# ---- up to 64 rows of x: the kernel that streams W once (mode 5; mode 0 picks it by itself) ----
+
+@pytest.mark.parametrize("kind", ["i8", "f16"])
+@pytest.mark.parametrize("M", [2, 7, 16, 17, 33, 48, 64])
+@pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (130, 576), (131, 64), (16, 64), (1000, 1024), (20000, 128)])
+def test_streaming_gemm_few_rows(queue, kind, M, N, K):
+    print(f"{kind} streaming gemm M={M} N={N} K={K}", flush=True)
+    W, X = synth_w(1700 + N, N, K), synth_x(1800 + M, M, K)
+    plan = []
+    if kind == "i8":
+        q, s = mil.quantize_int8(W)
+        got = _gemm(queue, M, N, K, X, q, s, "i8", 5, plan)
+        want = O.gemm_i8(X, q, s.view(np.uint16))
+    else:
+        got = _gemm(queue, M, N, K, X, W, None, "f16", 5, plan)
+        want = O.gemm_f16(X, W)
+    kernel, rows, slices = plan[0]
+    assert kernel == 4 and rows == 16 * ((M + 15) // 16) and slices in (1, 2, 4, 8)
+    assert_tolerance(got.view(np.float16), want.view(np.float16))
+    assert _ulp_apart(got, want).max() <= 1
+    assert np.mean(got == want) > 0.99
+
+
+def test_streaming_gemm_is_the_choice_for_a_few_rows_and_refuses_more_than_64(queue):
+    N, K = 1024, 512
+    W = synth_w(1900, N, K)
+    q, s = mil.quantize_int8(W)
+    for M, kernel in ((16, 4), (32, 4), (33, None), (64, None), (65, None)):
+        plan = []
+        _gemm(queue, M, N, K, synth_x(1901, M, K), q, s, "i8", 0, plan)
+        assert (plan[0][0] == 4) == (kernel == 4), plan
+    xb, wb, sb = mil.Buffer.from_host(synth_x(1902, 65, K)), mil.Buffer.from_host(q), mil.Buffer.from_host(s)
+    ob = mil.Buffer(65 * N * 2)
+    assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+    mil.lib().mi_set_gemm_mode(5)
+    try:
+        assert not mil.pytorch_linear(queue, 65, N, K, xb, wb, ob)      # mode 5 has no kernel for 65 rows
+    finally:
+        mil.lib().mi_set_gemm_mode(0)
+        mil.nnopt_unregister_weight(wb)
+
+
+@pytest.mark.parametrize("kind", ["i8", "f16"])
+def test_streaming_gemm_exact_on_integer_data_and_indices(queue, kind):
+    """Small integers: every sum is exact whatever the order, so the result is integer arithmetic's
+    (a wrong pairing of the two operands' K positions or of rows and columns cannot hide in a
+    tolerance); then unit rows of x, which must pick dequantised columns of W."""
+    rng = np.random.default_rng(11)
+    for (M, N, K) in ((64, 528, 1024), (23, 131, 4864), (16, 4864, 896)):
+        X = rng.integers(-3, 4, (M, K)).astype(np.float16)
+        if kind == "i8":
+            q = rng.integers(-127, 128, (N, K)).astype(np.int8)
+            s = (2.0 ** rng.integers(-10, -6, N)).astype(np.float16)
+            got = _gemm(queue, M, N, K, X, q, s, "i8", 5)
+            want = ((X.astype(np.int64) @ q.astype(np.int64).T).astype(np.float64) * s.astype(np.float64)).astype(np.float16)
+        else:
+            W = rng.integers(-8, 9, (N, K)).astype(np.float16)
+            got = _gemm(queue, M, N, K, X, W, None, "f16", 5)
+            want = (X.astype(np.int64) @ W.astype(np.int64).T).astype(np.float16)
+        assert np.array_equal(got.view(np.float16), want), (M, N, K)
+    M, N, K = 64, 320, 896
+    W = synth_w(1910, N, K)
+    ks = (np.arange(M) * 37 + 5) % K
+    X = np.zeros((M, K), np.float16)
+    X[np.arange(M), ks] = 1.0
+    if kind == "i8":
+        q, s = mil.quantize_int8(W)
+        got = _gemm(queue, M, N, K, X, q, s, "i8", 5).view(np.float16)
+        want = (q[:, ks].T.astype(np.float32) * s.astype(np.float32)[None, :]).astype(np.float16)
+    else:
+        got = _gemm(queue, M, N, K, X, W, None, "f16", 5).view(np.float16)
+        want = W[:, ks].T
+    assert np.array_equal(got, want)
+
+
+def test_streaming_gemm_repeats_identically(queue):
+    """25 launches of a shape whose K is shared by eight wavefronts per strip: identical results
+    (the slices' sums meet in LDS and are added in slice order, not in order of arrival)."""
+    M, N, K = 48, 896, 4864
+    W, X = synth_w(1940, N, K), synth_x(1941, M, K)
+    q, s = mil.quantize_int8(W)
+    xb, wb, sb = mil.Buffer.from_host(X), mil.Buffer.from_host(q), mil.Buffer.from_host(s)
+    assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+    outs = [mil.Buffer(M * N * 2) for _ in range(25)]
+    mil.lib().mi_set_gemm_mode(5)
+    try:
+        assert mil.linear_plan(queue, M, N, K, xb, wb) == (4, 48, 8)
+        for ob in outs:
+            assert mil.pytorch_linear(queue, M, N, K, xb, wb, ob)
+        queue.finish()
+    finally:
+        mil.lib().mi_set_gemm_mode(0)
+    first = outs[0].read(np.uint16, (M, N))
+    assert_tolerance(first.view(np.float16), O.gemm_i8(X, q, s.view(np.uint16)).view(np.float16))
     for i, ob in enumerate(outs[1:]):
         assert np.array_equal(ob.read(np.uint16, (M, N)), first), f"launch {i + 1} differs from launch 0"
     mil.nnopt_unregister_weight(wb)
