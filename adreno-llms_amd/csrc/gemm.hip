@@ -866,7 +866,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemm_skinny(const uint16_t* __res
                                                            const uint8_t* __restrict__ W,
                                                            const uint16_t* __restrict__ scale,
                                                            uint16_t* __restrict__ out, int M, int N, int K, int ks,
-                                                           int logical_blocks) {
+                                                           int logical_blocks, float* __restrict__ partial) {
     constexpr bool F16 = KIND == WK_F16;
     constexpr int WV = F16 ? 2 : 1;                       // 16-byte loads of W per lane, strip and iteration
     constexpr int kWB = F16 ? 2 : 1;                      // bytes per weight
@@ -881,7 +881,11 @@ __global__ __launch_bounds__(64 * kWaves) void gemm_skinny(const uint16_t* __res
     const int i = lane & 15, c = lane >> 4;
     const int slice = wave % ks;
     const int nit = K / 64;
-    const int it0 = nit * slice / ks, it1 = nit * (slice + 1) / ks;
+    // K is cut over the blocks of the grid's y (then `partial` takes raw sums, one M x N matrix per y,
+    // for reduce_partials) and, inside a block, over ks wavefronts
+    const int b0 = nit * static_cast<int>(blockIdx.y) / static_cast<int>(gridDim.y);
+    const int b1 = nit * (static_cast<int>(blockIdx.y) + 1) / static_cast<int>(gridDim.y);
+    const int it0 = b0 + (b1 - b0) * slice / ks, it1 = b0 + (b1 - b0) * (slice + 1) / ks;
 
     if constexpr (XL) {
         const int per_row = K / 8;                       // 16-byte pieces per row
@@ -1040,6 +1044,23 @@ __global__ __launch_bounds__(64 * kWaves) void gemm_skinny(const uint16_t* __res
                 #pragma unroll
                 for (int r = 0; r < 4; ++r) s4[r] = __half2float(__ushort_as_half(scale[nq + r < N ? nq + r : N - 1]));
             }
+            if (partial) {
+                float* pout = partial + static_cast<size_t>(blockIdx.y) * M * N;
+                #pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    const int m = 16 * t + i;
+                    if (m >= M) continue;
+                    float* dst = pout + static_cast<size_t>(m) * N + nq;
+                    if ((N % 4) == 0 && nq + 3 < N) {
+                        *reinterpret_cast<float4*>(dst) = float4{acc[q][t][0], acc[q][t][1], acc[q][t][2], acc[q][t][3]};
+                    } else {
+                        #pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (nq + r < N) dst[r] = acc[q][t][r];
+                    }
+                }
+                continue;
+            }
             #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 const int m = 16 * t + i;
@@ -1066,40 +1087,55 @@ inline size_t lds_bytes(int mt, int K, bool xl, int ks) {
            (ks > 1 ? static_cast<size_t>(kWaves) * mt * 4 * 64 * 4 : 0);
 }
 
-struct Shape { int ks; bool xl; };
-// Slices of K per strip (1, 2, 4, 8: the fewest that give the chip four wavefronts per CU; measured
-// at 4864 x 896: 4 slices 4.5 us, 8 slices 6.7 us), x in LDS where it fits.  One strip per wavefront:
-// two and four (the kernel's SW) were measured slower at every shape tried (fewer wavefronts; the
-// reads of x they save are not the bound).
-inline Shape pick_shape(int M, int N, int K, int cus) {
+struct Shape { int ks; bool xl; int kb; };
+// Slices of K per strip inside a block (1, 2, 4, 8: the fewest that give the chip four wavefronts
+// per CU; measured at 4864 x 896: 4 slices 4.5 us, 8 slices 6.7 us), x in LDS where it fits, and
+// slices of K over blocks (kb) where one block per strip still leaves most CUs idle and what a
+// single CU can pull bounds the launch (896 x 4864: 56 strips): their sums go through the
+// workspace and a second launch adds them in order.  One strip per wavefront: two and four (the
+// kernel's SW) were measured slower at every shape tried (fewer wavefronts; the reads of x they
+// save are not the bound).
+inline Shape pick_shape(int M, int N, int K, int cus, size_t workspace_bytes) {
     const int mt = (M + 15) / 16;
     const long strips = (N + 15) / 16;
-    Shape sh{1, false};
+    Shape sh{1, false, 1};
     while (sh.ks < kWaves && strips * sh.ks < 4L * cus && K / 64 >= 2 * sh.ks) sh.ks *= 2;
-    sh.xl = lds_bytes(mt, K, true, sh.ks) <= kLdsLimit;
+    // (a block whose eight wavefronts share one strip reads every byte of x once either way: no LDS then)
+    sh.xl = sh.ks < kWaves && lds_bytes(mt, K, true, sh.ks) <= kLdsLimit;
+    if (sh.ks == kWaves) {
+        while (sh.kb < 8 && strips * sh.kb * 2 <= cus && K / 64 >= 2 * sh.ks * sh.kb * 2 &&
+               static_cast<double>(sh.kb) * 2 * M * N * 4 <= static_cast<double>(workspace_bytes))
+            sh.kb *= 2;
+    }
     return sh;
 }
 
 // Where the streaming kernel is the library's own choice (measured against the tiles above, int8,
-// warm weights): up to 32 rows of x with x in LDS (4864 x 896: 4.5 / 5.6 us at 16 / 32 rows against
-// 6.6 / 6.7 us; 48 rows tie, 64 rows lose, 7.6 against 6.8 us), up to 16 rows when x has to come
-// from the caches (896 x 4864: 10.0 against 12.1 us), and no more strips than stay resident at
-// once: an lm_head of 151 936 rows streams at 4.0 TB/s here (a wavefront loads a strip, waits,
-// multiplies) against 4.8 TB/s in the wide kernel.
-inline bool preferred(int M, int N, int K, int cus) {
-    const Shape sh = pick_shape(M, N, K, cus);
-    return M <= (sh.xl ? 32 : 16) && (N + 15) / 16 <= 16L * cus;
+// warm weights, us).  With x in LDS, or one strip per block: up to 48 rows (4864 x 896: 4.9 / 6.0 /
+// 7.0 at 16 / 32 / 48 rows against 8.0 for the 64 x 64 tiles, 8.4 against 7.4 at 64; 2560 x 1024: 4.4 /
+// 5.3 / 6.7 against 9.2 / 9.3 / 8.9, 7.7 against 7.3 at 64); up to 64 rows where K is cut over blocks
+// as well (896 x 4864: 7.1 / 8.3 / 10.8 at 16 / 32 / 64 rows against 12.1 / 11.0 / 11.9; 1024 x 4608: 7.3 /
+// 8.5 / 10.9 against 10 to 11.4).  With x from the caches and shared by several strips per block,
+// only up to 16 rows (8192 x 2048 at 48 rows: 28 us against 17).  And no more strips than stay
+// resident at once: an lm_head of 151 936 rows streams at 4.0 TB/s here (a wavefront loads a
+// strip, waits, multiplies) against 4.8 TB/s in the wide kernel.
+inline bool preferred(int M, int N, int K, int cus, size_t workspace_bytes) {
+    const Shape sh = pick_shape(M, N, K, cus, workspace_bytes);
+    const int rows = sh.xl || sh.ks == kWaves ? (sh.kb > 1 ? 64 : 48) : 16;
+    return M <= rows && (N + 15) / 16 <= 16L * cus;
 }
 
 // Estimated time (us), fitted to the same measurements.
-inline double estimate_us(int kind, int M, int N, int K, int cus) {
-    const Shape sh = pick_shape(M, N, K, cus);
+inline double estimate_us(int kind, int M, int N, int K, int cus, size_t workspace_bytes) {
+    const Shape sh = pick_shape(M, N, K, cus, workspace_bytes);
     const double w_bytes = static_cast<double>(N) * K * (kind == WK_F16 ? 2.0 : 1.0);
-    return sh.xl ? 3.75 + 0.035 * M + w_bytes / 8.0e6 : 5.5 + 0.22 * M + w_bytes / 8.0e6;
+    return sh.xl ? 3.75 + 0.035 * M + w_bytes / 8.0e6 : (sh.kb > 1 ? 5.4 : 3.6) + 0.07 * M + w_bytes / 8.0e6;
 }
 
 template <int KIND, int MT, int SW, bool XL>
-bool launch_one(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, int ks) {
+bool launch_one(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, Shape sh,
+                float* partial) {
+    const int ks = sh.ks;
     const long groups = ((N + 15) / 16 + SW - 1) / SW, per_block = kWaves / ks;
     const long logical = (groups + per_block - 1) / per_block;
     const size_t lds = lds_bytes(MT, K, XL, ks);
@@ -1115,31 +1151,44 @@ bool launch_one(hipStream_t s, int M, int N, int K, const void* x, const void* W
         const long resident = static_cast<long>(device_info().cus) * (per_cu < 1 ? 1 : per_cu);
         if (grid > resident) grid = resident;
     }
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(64 * kWaves), lds, s, static_cast<const uint16_t*>(x),
-                       static_cast<const uint8_t*>(W), static_cast<const uint16_t*>(scale), static_cast<uint16_t*>(out),
-                       M, N, K, ks, static_cast<int>(logical));
-    return MI_HIP_OK(hipGetLastError());
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid), static_cast<unsigned>(sh.kb)), dim3(64 * kWaves), lds, s,
+                       static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(W), static_cast<const uint16_t*>(scale),
+                       static_cast<uint16_t*>(out), M, N, K, ks, static_cast<int>(logical), sh.kb > 1 ? partial : nullptr);
+    if (!MI_HIP_OK(hipGetLastError())) return false;
+    if (sh.kb > 1) {
+        const long MN = static_cast<long>(M) * N;
+        hipLaunchKernelGGL(wide::reduce_partials, dim3(static_cast<unsigned>((MN / 4 + 256) / 256)), dim3(256), 0, s, partial,
+                           sh.kb, KIND == WK_I8 ? static_cast<const uint16_t*>(scale) : nullptr, static_cast<uint16_t*>(out),
+                           MN, N);
+        if (!MI_HIP_OK(hipGetLastError())) return false;
+    }
+    return true;
 }
 
 template <int KIND, int MT>
-bool launch_mt(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, Shape sh) {
-    return sh.xl ? launch_one<KIND, MT, 1, true>(s, M, N, K, x, W, scale, out, sh.ks)
-                 : launch_one<KIND, MT, 1, false>(s, M, N, K, x, W, scale, out, sh.ks);
+bool launch_mt(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, Shape sh,
+               float* partial) {
+    return sh.xl ? launch_one<KIND, MT, 1, true>(s, M, N, K, x, W, scale, out, sh, partial)
+                 : launch_one<KIND, MT, 1, false>(s, M, N, K, x, W, scale, out, sh, partial);
 }
 
 template <int KIND>
-bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, Shape sh) {
+bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, Shape sh,
+            void* workspace, size_t workspace_bytes) {
     if (M < 1 || M > kMaxM || !(sh.ks == 1 || sh.ks == 2 || sh.ks == 4 || sh.ks == 8) ||
-        lds_bytes((M + 15) / 16, K, sh.xl, sh.ks) > kLdsLimit) {
-        MI_ERROR_FMT("gemm: the streaming kernel takes up to %d rows of x, 1, 2, 4 or 8 slices of K and %zu bytes of LDS "
-                     "(M=%d K=%d, %d slices, x in LDS %d)", kMaxM, kLdsLimit, M, K, sh.ks, static_cast<int>(sh.xl));
+        lds_bytes((M + 15) / 16, K, sh.xl, sh.ks) > kLdsLimit || sh.kb < 1 || (sh.kb > 1 && sh.xl) ||
+        (sh.kb > 1 && (!workspace || static_cast<double>(sh.kb) * M * N * 4 > static_cast<double>(workspace_bytes)))) {
+        MI_ERROR_FMT("gemm: the streaming kernel takes up to %d rows of x, 1, 2, 4 or 8 slices of K per block, %zu bytes of LDS "
+                     "and a workspace for slices over blocks (M=%d K=%d, %d slices, x in LDS %d, %d slices over blocks, %zu bytes)",
+                     kMaxM, kLdsLimit, M, K, sh.ks, static_cast<int>(sh.xl), sh.kb, workspace_bytes);
         return false;
     }
+    auto* partial = static_cast<float*>(workspace);
     switch ((M + 15) / 16) {
-        case 1: return launch_mt<KIND, 1>(s, M, N, K, x, W, scale, out, sh);
-        case 2: return launch_mt<KIND, 2>(s, M, N, K, x, W, scale, out, sh);
-        case 3: return launch_mt<KIND, 3>(s, M, N, K, x, W, scale, out, sh);
-        default: return launch_mt<KIND, 4>(s, M, N, K, x, W, scale, out, sh);
+        case 1: return launch_mt<KIND, 1>(s, M, N, K, x, W, scale, out, sh, partial);
+        case 2: return launch_mt<KIND, 2>(s, M, N, K, x, W, scale, out, sh, partial);
+        case 3: return launch_mt<KIND, 3>(s, M, N, K, x, W, scale, out, sh, partial);
+        default: return launch_mt<KIND, 4>(s, M, N, K, x, W, scale, out, sh, partial);
     }
 }
 
@@ -1213,8 +1262,8 @@ double gemm_estimate_us(WeightKind kind, int M, int N, int K, size_t workspace_b
     if (wide_reaches(kind, M, N, K))
         wide::pick_shape(kind, terms, M, N, K, device_info().cus, workspace_bytes, &tm, &splits, &wide_us);
     if (kind == WK_Q4) return wide_us;
-    if (M <= skinny::kMaxM && skinny::preferred(M, N, K, device_info().cus))
-        return skinny::estimate_us(kind, M, N, K, device_info().cus);
+    if (M <= skinny::kMaxM && skinny::preferred(M, N, K, device_info().cus, workspace_bytes))
+        return skinny::estimate_us(kind, M, N, K, device_info().cus, workspace_bytes);
     const double tiled_us = tiled_estimate_us(M, N, K);
     return wide_us < tiled_us ? wide_us : tiled_us;
 }
@@ -1239,8 +1288,9 @@ GemmPlan plan_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, size_t w
         return p;
     }
     // int8 and fp16, a few rows of x: the streaming kernel (mode 5 asks for it by name, up to 64 rows)
-    if (M <= skinny::kMaxM && (mode == 5 || (mode == 0 && skinny::preferred(M, N, K, cus)))) {
-        p.kernel = 4; p.tile_rows = 16 * ((M + 15) / 16); p.k_slices = skinny::pick_shape(M, N, K, cus).ks;
+    if (M <= skinny::kMaxM && (mode == 5 || (mode == 0 && skinny::preferred(M, N, K, cus, workspace_bytes)))) {
+        const skinny::Shape sh = skinny::pick_shape(M, N, K, cus, workspace_bytes);
+        p.kernel = 4; p.tile_rows = 16 * ((M + 15) / 16); p.k_slices = sh.ks * sh.kb;
         return p;
     }
     if (mode == 5) return p;
@@ -1284,8 +1334,11 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
             return wide::launch_any<WK_I8, 1>(tm, s, M, N, K, x, W, scale, out, partial, ws_bytes, p.k_slices);
         }
         case 4:
-            return kind == WK_F16 ? skinny::launch<WK_F16>(s, M, N, K, x, W, scale, out, skinny::pick_shape(M, N, K, device_info().cus))
-                                  : skinny::launch<WK_I8>(s, M, N, K, x, W, scale, out, skinny::pick_shape(M, N, K, device_info().cus));
+        {
+            const skinny::Shape sh = skinny::pick_shape(M, N, K, device_info().cus, ws_bytes);
+            return kind == WK_F16 ? skinny::launch<WK_F16>(s, M, N, K, x, W, scale, out, sh, workspace, ws_bytes)
+                                  : skinny::launch<WK_I8>(s, M, N, K, x, W, scale, out, sh, workspace, ws_bytes);
+        }
         case 2: return launch_tile<64, 64, 32, 32>(s, kind, M, N, K, x, W, scale, out);
         case 3: return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);
         default:

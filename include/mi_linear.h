@@ -174,8 +174,8 @@ int   mi_graph_destroy(void* graph);
  * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel (int8 and fp16
  * weights; fails for Q4), 3 = the wide kernel, 10 + t (t = 1..5) = the wide kernel with 32 t
  * rows of x per block, 5 = the streaming kernel for up to 64 rows of x (int8 and fp16 weights, which
- * take it by themselves in mode 0 up to 32 rows where it is the faster one; fails for more than 64
- * rows; Q4 weights take the wide kernel).
+ * take it by themselves in mode 0 up to 48 or 64 rows, depending on the shape, where it is the
+ * faster one; fails for more than 64 rows; Q4 weights take the wide kernel).
  * Q4 weights: a weight q * scale (4 and 11 significant bits) is not an fp16 number in general.
  * Every mode but 4 feeds it to the matrix cores exactly, as two fp16 terms q * hi + q * lo with
  * scale = hi + lo, and stays within one fp16 step of the batched GEMV.  Mode 4 = as 0, but each
@@ -202,8 +202,9 @@ int mi_stream_set_modes(void* stream, int gemv_mode, int gemm_mode);
  * row of x), 1 = the wide MFMA kernel with *tile_rows rows of x per block and K cut into
  * *k_slices slices (more than one slice: fp32 partial sums in the stream's workspace and a
  * reduction launch), 2 / 3 = the 64 x 64 / 128 x 128 tile kernel, 4 = the streaming kernel for up
- * to 64 rows of x (*tile_rows = M rounded up to 16, *k_slices = wavefronts of a block that share
- * one strip of 16 rows of W), -1 = bad arguments.  For tests and tuning; tile_rows and k_slices
+ * to 64 rows of x (*tile_rows = M rounded up to 16, *k_slices = wavefronts, over one or several
+ * blocks, that share one strip of 16 rows of W; slices over several blocks also end in a reduction
+ * launch), -1 = bad arguments.  For tests and tuning; tile_rows and k_slices
  * may be NULL. */
 int mi_linear_plan(void* stream, int M, int N, int K, const void* x, const void* W, int* tile_rows, int* k_slices);
 
