@@ -871,7 +871,8 @@ __global__ __launch_bounds__(64 * kWaves) void gemm_skinny(const uint16_t* __res
     constexpr int WV = F16 ? 2 : 1;                       // 16-byte loads of W per lane, strip and iteration
     constexpr int kWB = F16 ? 2 : 1;                      // bytes per weight
     constexpr int kPerIt = 4 * SW * WV + (XL ? 0 : 8 * MT);   // registers one iteration's operands take in a buffer
-    constexpr int kChunk = 64 / kPerIt < 1 ? 1 : 64 / kPerIt > 8 ? 8 : 64 / kPerIt;   // iterations per register buffer
+    constexpr int kBudget = F16 ? 40 : 48;                // registers per buffer (with 64 the fp16 instances spill)
+    constexpr int kChunk = kBudget / kPerIt < 1 ? 1 : kBudget / kPerIt > 8 ? 8 : kBudget / kPerIt;   // iterations per buffer
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t xrow = XL ? static_cast<uint32_t>(K) * 2u + 16u : 0u;              // bytes per row of x in LDS
     float* red = reinterpret_cast<float*>(lds + 16u * MT * xrow);                     // [kWaves][MT][4][64]
