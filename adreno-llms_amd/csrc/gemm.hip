@@ -861,16 +861,22 @@ constexpr int kWaves = 8;                // wavefronts per block
 // blocks then live long and walk over the strips.  Without XL (x too large for LDS) the fragments
 // come from the caches with the weights, 2 MT / SW bytes per byte of W, and the L1's few requests
 // in flight bound the rate: that form only pays for a few rows of x at a long K.
-template <int KIND, int MT, int SW, bool XL>
+// Q4 weights: an iteration is 128 values of K, of which a lane holds 32, exactly one scale block (16
+// bytes of nibbles and one scale per lane and iteration); the weights enter the matrix cores as
+// q * scale, exactly, in TERMS = 2 fp16 terms (scale = hi + lo with 7 and 4 significant bits, as in
+// the wide kernel), or rounded to fp16 once with TERMS = 1.
+template <int KIND, int MT, int SW, bool XL, int TERMS>
 __global__ __launch_bounds__(64 * kWaves) void gemm_skinny(const uint16_t* __restrict__ X,
                                                            const uint8_t* __restrict__ W,
                                                            const uint16_t* __restrict__ scale,
                                                            uint16_t* __restrict__ out, int M, int N, int K, int ks,
                                                            int logical_blocks, float* __restrict__ partial) {
-    constexpr bool F16 = KIND == WK_F16;
+    constexpr bool F16 = KIND == WK_F16, Q4 = KIND == WK_Q4;
     constexpr int WV = F16 ? 2 : 1;                       // 16-byte loads of W per lane, strip and iteration
-    constexpr int kWB = F16 ? 2 : 1;                      // bytes per weight
-    constexpr int kPerIt = 4 * SW * WV + (XL ? 0 : 8 * MT);   // registers one iteration's operands take in a buffer
+    constexpr int kWB = F16 ? 2 : 1;                      // bytes of a row of W per 64 bytes of an iteration's weights / 64
+    constexpr int kItK = Q4 ? 128 : 64;                   // values of K per iteration
+    constexpr int XE = kItK / 32;                         // 16-byte pieces of x per lane and iteration = MFMAs per x tile and term
+    constexpr int kPerIt = (4 * WV + (Q4 ? 1 : 0)) * SW + (XL ? 0 : 4 * XE * MT);   // registers one iteration's operands take in a buffer
     constexpr int kBudget = F16 ? 40 : 48;                // registers per buffer (with 64 the fp16 instances spill)
     constexpr int kChunk = kBudget / kPerIt < 1 ? 1 : kBudget / kPerIt > 8 ? 8 : kBudget / kPerIt;   // iterations per buffer
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -881,7 +887,8 @@ __global__ __launch_bounds__(64 * kWaves) void gemm_skinny(const uint16_t* __res
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, c = lane >> 4;
     const int slice = wave % ks;
-    const int nit = K / 64;
+    const int nit = (K + kItK - 1) / kItK;               // (Q4 at K = 64 mod 128: the upper half of the lanes sits out the last one)
+    const size_t wrowb = Q4 ? static_cast<size_t>(K) / 2 : static_cast<size_t>(K) * kWB;   // bytes of a row of W
     // K is cut over the blocks of the grid's y (then `partial` takes raw sums, one M x N matrix per y,
     // for reduce_partials) and, inside a block, over ks wavefronts
     const int b0 = nit * static_cast<int>(blockIdx.y) / static_cast<int>(gridDim.y);
@@ -902,18 +909,20 @@ __global__ __launch_bounds__(64 * kWaves) void gemm_skinny(const uint16_t* __res
     #pragma unroll
     for (int t = 0; t < MT; ++t) {
         const int m = 16 * t + i < M ? 16 * t + i : M - 1;
-        xp[t] = reinterpret_cast<const uint8_t*>(X) + static_cast<size_t>(m) * K * 2 + c * 32;
+        xp[t] = reinterpret_cast<const uint8_t*>(X) + static_cast<size_t>(m) * K * 2 + c * (16 * XE);
     }
-    const uint32_t xl = (16u * 0 + i) * xrow + c * 32u;  // with XL: this lane's row of the first x tile in LDS
+    const uint32_t xl = (16u * 0 + i) * xrow + c * (16u * XE);  // with XL: this lane's row of the first x tile in LDS
     const bool cols4 = (N % 4) == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0;
 
     for (int lb = blockIdx.x; lb < logical_blocks; lb += gridDim.x) {     // (the same trips for the whole block)
         const int group = lb * (kWaves / ks) + wave / ks;                 // group: SW consecutive strips
         const uint8_t* wp[SW];
+        [[maybe_unused]] const uint16_t* sp[SW];                          // Q4: the row's block scales, this lane's first
         #pragma unroll
         for (int q = 0; q < SW; ++q) {
             const int row = 16 * (group * SW + q) + i;                    // rows past N are read as the last row
-            wp[q] = W + static_cast<size_t>(row < N ? row : N - 1) * K * kWB + c * 16 * WV;
+            wp[q] = W + static_cast<size_t>(row < N ? row : N - 1) * wrowb + c * 16 * WV;
+            if constexpr (Q4) sp[q] = scale + static_cast<size_t>(row < N ? row : N - 1) * (K / 32) + c;
         }
         floatx4 acc[SW][MT];
         #pragma unroll
@@ -922,7 +931,8 @@ __global__ __launch_bounds__(64 * kWaves) void gemm_skinny(const uint16_t* __res
             for (int t = 0; t < MT; ++t) acc[q][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 
         u32x4 wb[2][kChunk][SW][WV];
-        [[maybe_unused]] u32x4 xb[2][XL ? 1 : kChunk][XL ? 1 : MT][2];
+        [[maybe_unused]] uint16_t sb[2][kChunk][SW];
+        [[maybe_unused]] u32x4 xb[2][XL ? 1 : kChunk][XL ? 1 : MT][XE];
         // `full`: kChunk iterations whatever the slice's end (the caller knows they exist); the number
         // of requests is then a constant, and only then can the wait before a buffer is multiplied
         // leave the other buffer's requests in flight
@@ -933,54 +943,84 @@ __global__ __launch_bounds__(64 * kWaves) void gemm_skinny(const uint16_t* __res
                 if constexpr (!decltype(fullc)::value) {
                     if (it >= it1) break;
                 }
+                // (Q4, K = 64 mod 128: a lane without weights in the last iteration asks for the start of its rows)
+                [[maybe_unused]] const bool mine = !Q4 || kItK * it + 32 * c < K;
                 if constexpr (!XL) {
                     #pragma unroll
                     for (int t = 0; t < MT; ++t)
                         #pragma unroll
-                        for (int e = 0; e < 2; ++e)
-                            xb[b][u][t][e] = reinterpret_cast<const u32x4*>(xp[t] + static_cast<size_t>(it) * 128)[e];
+                        for (int e = 0; e < XE; ++e)
+                            xb[b][u][t][e] = reinterpret_cast<const u32x4*>(
+                                xp[t] + (mine ? static_cast<ptrdiff_t>(it) * (2 * kItK) : -static_cast<ptrdiff_t>(c) * (16 * XE)))[e];
                 }
                 #pragma unroll
-                for (int q = 0; q < SW; ++q)
+                for (int q = 0; q < SW; ++q) {
                     #pragma unroll
                     for (int v = 0; v < WV; ++v)
-                        wb[b][u][q][v] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp[q] + static_cast<size_t>(it) * 64 * kWB) + v);
+                        wb[b][u][q][v] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+                            wp[q] + (mine ? static_cast<ptrdiff_t>(it) * 64 * kWB : -static_cast<ptrdiff_t>(c) * 16 * WV)) + v);
+                    if constexpr (Q4) sb[b][u][q] = sp[q][mine ? 4 * it : -c];
+                }
             }
         };
         auto multiply = [&](int b, int j0) {
             #pragma unroll
             for (int u = 0; u < kChunk; ++u) {
-                if (j0 + u < it1) {
-                    half8 xf[MT][2];
+                const int it = j0 + u;
+                if (it < it1) {
+                    [[maybe_unused]] const bool mine = !Q4 || kItK * it + 32 * c < K;
+                    half8 xf[MT][XE];
                     #pragma unroll
                     for (int t = 0; t < MT; ++t)
                         #pragma unroll
-                        for (int e = 0; e < 2; ++e) {
+                        for (int e = 0; e < XE; ++e) {
                             if constexpr (XL)
-                                xf[t][e] = *reinterpret_cast<const half8*>(lds + xl + 16u * t * xrow + (j0 + u) * 128 + 16 * e);
+                                xf[t][e] = *reinterpret_cast<const half8*>(
+                                    lds + xl + 16u * t * xrow + (mine ? it * (2 * kItK) : -c * (16 * XE)) + 16 * e);
                             else
                                 xf[t][e] = __builtin_bit_cast(half8, xb[b][u][t][e]);
                         }
                     #pragma unroll
                     for (int q = 0; q < SW; ++q) {
-                        half8 a[2];
+                        half8 a[TERMS][XE];
                         if constexpr (F16) {
-                            a[0] = __builtin_bit_cast(half8, wb[b][u][q][0]);
-                            a[1] = __builtin_bit_cast(half8, wb[b][u][q][1]);
+                            a[0][0] = __builtin_bit_cast(half8, wb[b][u][q][0]);
+                            a[0][1] = __builtin_bit_cast(half8, wb[b][u][q][1]);
+                        } else if constexpr (Q4) {
+                            // a lane that sits the iteration out multiplies by a scale of zero
+                            const uint32_t s1 = mine ? sb[b][u][q] : 0u;
+                            const uint32_t sboth = s1 | (s1 << 16);
+                            __half2 st[TERMS];
+                            if constexpr (TERMS == 2) {
+                                st[0] = __builtin_bit_cast(__half2, sboth & 0xFFF0FFF0u);
+                                st[1] = __hsub2(__builtin_bit_cast(__half2, sboth), st[0]);
+                            } else {
+                                st[0] = __builtin_bit_cast(__half2, sboth);
+                            }
+                            #pragma unroll
+                            for (int e = 0; e < XE; ++e) {
+                                const uint32_t v = wb[b][u][q][0][e];
+                                #pragma unroll
+                                for (int z = 0; z < TERMS; ++z)
+                                    a[z][e] = __builtin_bit_cast(half8, u32x4{q4x2_to_h2<0>(v, st[z]), q4x2_to_h2<1>(v, st[z]),
+                                                                              q4x2_to_h2<2>(v, st[z]), q4x2_to_h2<3>(v, st[z])});
+                            }
                         } else {
                             uint32_t h[8];
                             i8x4_to_h4(wb[b][u][q][0].x, h[0], h[1]);
                             i8x4_to_h4(wb[b][u][q][0].y, h[2], h[3]);
                             i8x4_to_h4(wb[b][u][q][0].z, h[4], h[5]);
                             i8x4_to_h4(wb[b][u][q][0].w, h[6], h[7]);
-                            a[0] = __builtin_bit_cast(half8, u32x4{h[0], h[1], h[2], h[3]});
-                            a[1] = __builtin_bit_cast(half8, u32x4{h[4], h[5], h[6], h[7]});
+                            a[0][0] = __builtin_bit_cast(half8, u32x4{h[0], h[1], h[2], h[3]});
+                            a[0][1] = __builtin_bit_cast(half8, u32x4{h[4], h[5], h[6], h[7]});
                         }
                         #pragma unroll
                         for (int t = 0; t < MT; ++t)
                             #pragma unroll
-                            for (int e = 0; e < 2; ++e)
-                                acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[e], xf[t][e], acc[q][t], 0, 0, 0);
+                            for (int z = 0; z < TERMS; ++z)
+                                #pragma unroll
+                                for (int e = 0; e < XE; ++e)
+                                    acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[z][e], xf[t][e], acc[q][t], 0, 0, 0);
                     }
                 }
             }
@@ -1096,15 +1136,16 @@ struct Shape { int ks; bool xl; int kb; };
 // workspace and a second launch adds them in order.  One strip per wavefront: two and four (the
 // kernel's SW) were measured slower at every shape tried (fewer wavefronts; the reads of x they
 // save are not the bound).
-inline Shape pick_shape(int M, int N, int K, int cus, size_t workspace_bytes) {
+inline Shape pick_shape(int kind, int M, int N, int K, int cus, size_t workspace_bytes) {
     const int mt = (M + 15) / 16;
     const long strips = (N + 15) / 16;
+    const int its = kind == WK_Q4 ? (K + 127) / 128 : K / 64;        // iterations over K
     Shape sh{1, false, 1};
-    while (sh.ks < kWaves && strips * sh.ks < 4L * cus && K / 64 >= 2 * sh.ks) sh.ks *= 2;
+    while (sh.ks < kWaves && strips * sh.ks < 4L * cus && its >= 2 * sh.ks) sh.ks *= 2;
     // (a block whose eight wavefronts share one strip reads every byte of x once either way: no LDS then)
     sh.xl = sh.ks < kWaves && lds_bytes(mt, K, true, sh.ks) <= kLdsLimit;
     if (sh.ks == kWaves) {
-        while (sh.kb < 8 && strips * sh.kb * 2 <= cus && K / 64 >= 2 * sh.ks * sh.kb * 2 &&
+        while (sh.kb < 8 && strips * sh.kb * 2 <= cus && its >= 2 * sh.ks * sh.kb * 2 &&
                static_cast<double>(sh.kb) * 2 * M * N * 4 <= static_cast<double>(workspace_bytes))
             sh.kb *= 2;
     }
@@ -1120,27 +1161,30 @@ inline Shape pick_shape(int M, int N, int K, int cus, size_t workspace_bytes) {
 // only up to 16 rows (8192 x 2048 at 48 rows: 28 us against 17).  And no more strips than stay
 // resident at once: an lm_head of 151 936 rows streams at 4.0 TB/s here (a wavefront loads a
 // strip, waits, multiplies) against 4.8 TB/s in the wide kernel.
-inline bool preferred(int M, int N, int K, int cus, size_t workspace_bytes) {
-    const Shape sh = pick_shape(M, N, K, cus, workspace_bytes);
-    const int rows = sh.xl || sh.ks == kWaves ? (sh.kb > 1 ? 64 : 48) : 16;
+inline bool preferred(int kind, int M, int N, int K, int cus, size_t workspace_bytes) {
+    const Shape sh = pick_shape(kind, M, N, K, cus, workspace_bytes);
+    int rows = sh.xl || sh.ks == kWaves ? (sh.kb > 1 ? 64 : 48) : 16;
+    // Q4 with x from the caches holds twice the x per iteration in registers: 48 rows spill a little,
+    // 64 a lot (896 x 4864: 10.5 / 13.7 / 26.8 us at 32 / 48 / 64 rows)
+    if (kind == WK_Q4 && !sh.xl && rows > 32) rows = 32;
     return M <= rows && (N + 15) / 16 <= 16L * cus;
 }
 
 // Estimated time (us), fitted to the same measurements.
 inline double estimate_us(int kind, int M, int N, int K, int cus, size_t workspace_bytes) {
-    const Shape sh = pick_shape(M, N, K, cus, workspace_bytes);
-    const double w_bytes = static_cast<double>(N) * K * (kind == WK_F16 ? 2.0 : 1.0);
+    const Shape sh = pick_shape(kind, M, N, K, cus, workspace_bytes);
+    const double w_bytes = static_cast<double>(N) * K * (kind == WK_F16 ? 2.0 : kind == WK_Q4 ? 0.5625 : 1.0);
     return sh.xl ? 3.75 + 0.035 * M + w_bytes / 8.0e6 : (sh.kb > 1 ? 5.4 : 3.6) + 0.07 * M + w_bytes / 8.0e6;
 }
 
-template <int KIND, int MT, int SW, bool XL>
+template <int KIND, int MT, int SW, bool XL, int TERMS>
 bool launch_one(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, Shape sh,
                 float* partial) {
     const int ks = sh.ks;
     const long groups = ((N + 15) / 16 + SW - 1) / SW, per_block = kWaves / ks;
     const long logical = (groups + per_block - 1) / per_block;
     const size_t lds = lds_bytes(MT, K, XL, ks);
-    auto* kern = gemm_skinny<KIND, MT, SW, XL>;
+    auto* kern = gemm_skinny<KIND, MT, SW, XL, TERMS>;
     if (lds > 65536 &&
         !MI_ONCE_OK(MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsLimit)))))
@@ -1166,14 +1210,14 @@ bool launch_one(hipStream_t s, int M, int N, int K, const void* x, const void* W
     return true;
 }
 
-template <int KIND, int MT>
+template <int KIND, int MT, int TERMS>
 bool launch_mt(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, Shape sh,
                float* partial) {
-    return sh.xl ? launch_one<KIND, MT, 1, true>(s, M, N, K, x, W, scale, out, sh, partial)
-                 : launch_one<KIND, MT, 1, false>(s, M, N, K, x, W, scale, out, sh, partial);
+    return sh.xl ? launch_one<KIND, MT, 1, true, TERMS>(s, M, N, K, x, W, scale, out, sh, partial)
+                 : launch_one<KIND, MT, 1, false, TERMS>(s, M, N, K, x, W, scale, out, sh, partial);
 }
 
-template <int KIND>
+template <int KIND, int TERMS>
 bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out, Shape sh,
             void* workspace, size_t workspace_bytes) {
     if (M < 1 || M > kMaxM || !(sh.ks == 1 || sh.ks == 2 || sh.ks == 4 || sh.ks == 8) ||
@@ -1186,10 +1230,10 @@ bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, co
     }
     auto* partial = static_cast<float*>(workspace);
     switch ((M + 15) / 16) {
-        case 1: return launch_mt<KIND, 1>(s, M, N, K, x, W, scale, out, sh, partial);
-        case 2: return launch_mt<KIND, 2>(s, M, N, K, x, W, scale, out, sh, partial);
-        case 3: return launch_mt<KIND, 3>(s, M, N, K, x, W, scale, out, sh, partial);
-        default: return launch_mt<KIND, 4>(s, M, N, K, x, W, scale, out, sh, partial);
+        case 1: return launch_mt<KIND, 1, TERMS>(s, M, N, K, x, W, scale, out, sh, partial);
+        case 2: return launch_mt<KIND, 2, TERMS>(s, M, N, K, x, W, scale, out, sh, partial);
+        case 3: return launch_mt<KIND, 3, TERMS>(s, M, N, K, x, W, scale, out, sh, partial);
+        default: return launch_mt<KIND, 4, TERMS>(s, M, N, K, x, W, scale, out, sh, partial);
     }
 }
 
@@ -1262,9 +1306,9 @@ double gemm_estimate_us(WeightKind kind, int M, int N, int K, size_t workspace_b
     int tm = 1, splits = 1;
     if (wide_reaches(kind, M, N, K))
         wide::pick_shape(kind, terms, M, N, K, device_info().cus, workspace_bytes, &tm, &splits, &wide_us);
-    if (kind == WK_Q4) return wide_us;
-    if (M <= skinny::kMaxM && skinny::preferred(M, N, K, device_info().cus, workspace_bytes))
+    if (M <= skinny::kMaxM && skinny::preferred(kind, M, N, K, device_info().cus, workspace_bytes))
         return skinny::estimate_us(kind, M, N, K, device_info().cus, workspace_bytes);
+    if (kind == WK_Q4) return wide_us;
     const double tiled_us = tiled_estimate_us(M, N, K);
     return wide_us < tiled_us ? wide_us : tiled_us;
 }
@@ -1276,12 +1320,19 @@ GemmPlan plan_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, size_t w
     const bool wide_fits = wide_reaches(kind, M, N, K);
     int tm = 1, splits = 1;
     if (kind == WK_Q4) {
-        // Q4 weights have the wide kernel only; modes 3 and 11..15 pin it to one slice of K.
+        // Q4 weights have the streaming kernel (a few rows of x; mode 5 asks for it by name) and the
+        // wide kernel; modes 3 and 11..15 pin the latter to one slice of K.
         // Mode 4 feeds every weight as the single fp16 number nearest to q * scale (half the
         // MFMAs, an error of up to 2^-12 sum |w x|); all other modes feed q * scale exactly, as
         // two fp16 terms.
-        if (!wide_fits || mode == 2) return p;
+        if (mode == 2) return p;
         p.terms = mode == 4 ? 1 : 2;
+        if (M <= skinny::kMaxM && (mode == 5 || ((mode == 0 || mode == 4) && skinny::preferred(WK_Q4, M, N, K, cus, workspace_bytes)))) {
+            const skinny::Shape sh = skinny::pick_shape(WK_Q4, M, N, K, cus, workspace_bytes);
+            p.kernel = 4; p.tile_rows = 16 * ((M + 15) / 16); p.k_slices = sh.ks * sh.kb;
+            return p;
+        }
+        if (!wide_fits || mode == 5) return p;
         const bool may_slice = mode == 0 || mode == 4;
         wide::pick_shape(WK_Q4, p.terms, M, N, K, cus, may_slice ? workspace_bytes : 0, &tm, &splits, nullptr);
         if (mode >= 11 && mode <= 15) tm = mode - 10;
@@ -1289,8 +1340,8 @@ GemmPlan plan_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, size_t w
         return p;
     }
     // int8 and fp16, a few rows of x: the streaming kernel (mode 5 asks for it by name, up to 64 rows)
-    if (M <= skinny::kMaxM && (mode == 5 || (mode == 0 && skinny::preferred(M, N, K, cus, workspace_bytes)))) {
-        const skinny::Shape sh = skinny::pick_shape(M, N, K, cus, workspace_bytes);
+    if (M <= skinny::kMaxM && (mode == 5 || (mode == 0 && skinny::preferred(kind, M, N, K, cus, workspace_bytes)))) {
+        const skinny::Shape sh = skinny::pick_shape(kind, M, N, K, cus, workspace_bytes);
         p.kernel = 4; p.tile_rows = 16 * ((M + 15) / 16); p.k_slices = sh.ks * sh.kb;
         return p;
     }
@@ -1336,9 +1387,12 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
         }
         case 4:
         {
-            const skinny::Shape sh = skinny::pick_shape(M, N, K, device_info().cus, ws_bytes);
-            return kind == WK_F16 ? skinny::launch<WK_F16>(s, M, N, K, x, W, scale, out, sh, workspace, ws_bytes)
-                                  : skinny::launch<WK_I8>(s, M, N, K, x, W, scale, out, sh, workspace, ws_bytes);
+            const skinny::Shape sh = skinny::pick_shape(kind, M, N, K, device_info().cus, ws_bytes);
+            if (kind == WK_Q4)
+                return p.terms == 1 ? skinny::launch<WK_Q4, 1>(s, M, N, K, x, W, scale, out, sh, workspace, ws_bytes)
+                                    : skinny::launch<WK_Q4, 2>(s, M, N, K, x, W, scale, out, sh, workspace, ws_bytes);
+            return kind == WK_F16 ? skinny::launch<WK_F16, 1>(s, M, N, K, x, W, scale, out, sh, workspace, ws_bytes)
+                                  : skinny::launch<WK_I8, 1>(s, M, N, K, x, W, scale, out, sh, workspace, ws_bytes);
         }
         case 2: return launch_tile<64, 64, 32, 32>(s, kind, M, N, K, x, W, scale, out);
         case 3: return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);

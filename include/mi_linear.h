@@ -173,9 +173,9 @@ int   mi_graph_destroy(void* graph);
  * 2, 3 and 11..15 = as 0 with the kernel choice pinned (tests and tuning: results stay within
  * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel (int8 and fp16
  * weights; fails for Q4), 3 = the wide kernel, 10 + t (t = 1..5) = the wide kernel with 32 t
- * rows of x per block, 5 = the streaming kernel for up to 64 rows of x (int8 and fp16 weights, which
- * take it by themselves in mode 0 up to 48 or 64 rows, depending on the shape, where it is the
- * faster one; fails for more than 64 rows; Q4 weights take the wide kernel).
+ * rows of x per block, 5 = the streaming kernel for up to 64 rows of x (every kind of weights takes
+ * it by itself in mode 0 up to 32 to 64 rows, depending on the shape, where it is the faster one;
+ * fails for more than 64 rows).
  * Q4 weights: a weight q * scale (4 and 11 significant bits) is not an fp16 number in general.
  * Every mode but 4 feeds it to the matrix cores exactly, as two fp16 terms q * hi + q * lo with
  * scale = hi + lo, and stays within one fp16 step of the batched GEMV.  Mode 4 = as 0, but each

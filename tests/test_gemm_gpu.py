@@ -158,10 +158,12 @@ def test_gemm_repeats_identically(queue, tile):
 
 # ---- up to 64 rows of x: the kernel that streams W once (mode 5; mode 0 picks it by itself) ----
 
-@pytest.mark.parametrize("kind", ["i8", "f16"])
+@pytest.mark.parametrize("kind", ["i8", "f16", "q4"])
 @pytest.mark.parametrize("M", [2, 7, 16, 17, 33, 48, 64])
-@pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (130, 576), (131, 64), (16, 64), (1000, 1024), (20000, 128)])
+@pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (130, 576), (131, 64), (16, 64), (1000, 1024), (20000, 128),
+                                 (520, 192), (1024, 4608)])
 def test_streaming_gemm_few_rows(queue, kind, M, N, K):
+    """(Q4: an iteration is 128 values of K; at K = 64, 192, 576 half of the lanes sit the last one out.)"""
     print(f"{kind} streaming gemm M={M} N={N} K={K}", flush=True)
     W, X = synth_w(1700 + N, N, K), synth_x(1800 + M, M, K)
     plan = []
@@ -169,6 +171,13 @@ def test_streaming_gemm_few_rows(queue, kind, M, N, K):
         q, s = mil.quantize_int8(W)
         got = _gemm(queue, M, N, K, X, q, s, "i8", 5, plan)
         want = O.gemm_i8(X, q, s.view(np.uint16))
+    elif kind == "q4":
+        p, s = mil.quantize_q4(W)
+        got = _gemm(queue, M, N, K, X, p, s, "q4", 5, plan)
+        want = O.gemm_q4(X, p, s.view(np.uint16))
+        wt = _q4_values(p).astype(np.float64) * np.repeat(s.astype(np.float64), 32, axis=1)
+        exact = (X.astype(np.float64) @ wt.T).astype(np.float16)
+        assert _ulp_apart(got, exact.view(np.uint16)).max() <= 1      # the weights entered exactly: one rounding from the true sum
     else:
         got = _gemm(queue, M, N, K, X, W, None, "f16", 5, plan)
         want = O.gemm_f16(X, W)
@@ -177,6 +186,17 @@ def test_streaming_gemm_few_rows(queue, kind, M, N, K):
     assert_tolerance(got.view(np.float16), want.view(np.float16))
     assert _ulp_apart(got, want).max() <= 1
     assert np.mean(got == want) > 0.99
+
+
+def _streaming_q4(queue, M, N, K, X, p, s, kind):
+    """Q4 through the streaming kernel: two exact terms (mode 5), or each weight rounded to fp16 once
+    (mode 4, at a shape where mode 4 takes the streaming kernel by itself)."""
+    if kind == "q4":
+        return _gemm(queue, M, N, K, X, p, s, "q4", 5)
+    plan = []
+    got = _gemm(queue, M, N, K, X, p, s, "q4", 4, plan)
+    assert plan[0][0] == 4, plan
+    return got
 
 
 def test_streaming_gemm_is_the_choice_for_a_few_rows_and_refuses_more_than_64(queue):
@@ -198,25 +218,32 @@ def test_streaming_gemm_is_the_choice_for_a_few_rows_and_refuses_more_than_64(qu
         mil.nnopt_unregister_weight(wb)
 
 
-@pytest.mark.parametrize("kind", ["i8", "f16"])
+@pytest.mark.parametrize("kind", ["i8", "f16", "q4", "q4_single_rounding"])
 def test_streaming_gemm_exact_on_integer_data_and_indices(queue, kind):
     """Small integers: every sum is exact whatever the order, so the result is integer arithmetic's
     (a wrong pairing of the two operands' K positions or of rows and columns cannot hide in a
     tolerance); then unit rows of x, which must pick dequantised columns of W."""
     rng = np.random.default_rng(11)
-    for (M, N, K) in ((64, 528, 1024), (23, 131, 4864), (16, 4864, 896)):
+    for (M, N, K) in ((32, 528, 1024), (23, 131, 4864), (16, 4864, 896)):
         X = rng.integers(-3, 4, (M, K)).astype(np.float16)
         if kind == "i8":
             q = rng.integers(-127, 128, (N, K)).astype(np.int8)
             s = (2.0 ** rng.integers(-10, -6, N)).astype(np.float16)
             got = _gemm(queue, M, N, K, X, q, s, "i8", 5)
             want = ((X.astype(np.int64) @ q.astype(np.int64).T).astype(np.float64) * s.astype(np.float64)).astype(np.float16)
+        elif kind.startswith("q4"):
+            # power-of-two block scales: q * scale is an fp16 number, every product and sum exact in either mode
+            p = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
+            s = (2.0 ** rng.integers(-6, -2, (N, K // 32))).astype(np.float16)
+            got = _streaming_q4(queue, M, N, K, X, p, s, kind)
+            wt = _q4_values(p).astype(np.float64) * np.repeat(s.astype(np.float64), 32, axis=1)
+            want = (X.astype(np.float64) @ wt.T).astype(np.float16)
         else:
             W = rng.integers(-8, 9, (N, K)).astype(np.float16)
             got = _gemm(queue, M, N, K, X, W, None, "f16", 5)
             want = (X.astype(np.int64) @ W.astype(np.int64).T).astype(np.float16)
         assert np.array_equal(got.view(np.float16), want), (M, N, K)
-    M, N, K = 64, 320, 896
+    M, N, K = 48, 320, 896
     W = synth_w(1910, N, K)
     ks = (np.arange(M) * 37 + 5) % K
     X = np.zeros((M, K), np.float16)
@@ -225,6 +252,11 @@ def test_streaming_gemm_exact_on_integer_data_and_indices(queue, kind):
         q, s = mil.quantize_int8(W)
         got = _gemm(queue, M, N, K, X, q, s, "i8", 5).view(np.float16)
         want = (q[:, ks].T.astype(np.float32) * s.astype(np.float32)[None, :]).astype(np.float16)
+    elif kind.startswith("q4"):
+        p, s = mil.quantize_q4(W)
+        got = _streaming_q4(queue, M, N, K, X, p, s, kind).view(np.float16)
+        # q * scale of column k, rounded to fp16 once (exact in two terms, the nearest fp16 in one: the same number)
+        want = (_q4_values(p)[:, ks].T.astype(np.float32) * s.astype(np.float32)[:, ks // 32].T).astype(np.float16)
     else:
         got = _gemm(queue, M, N, K, X, W, None, "f16", 5).view(np.float16)
         want = W[:, ks].T
