@@ -222,6 +222,22 @@ __device__ __forceinline__ Seg find_segment(const SegList& L, int rb) {
     return sg;
 }
 
+// The first 14 dwords of a kernel's arguments arrive in scalar registers with the wavefront (the
+// build asks for 16; two user registers go to the argument pointer itself); everything after them
+// is fetched by the kernel's first instructions, and the vector loads that depend on it wait for
+// that fetch.  So what the first loads need comes first, as plain arguments, in the order of need:
+// x, the first segment's N and the number of row batches, the first segment's W and scales, the
+// norm weights, the second segment's W and scales (null: one segment); y, which only the residual
+// load and the stores need, is the first to be fetched.  The SegList behind them holds the same and
+// the rest.
+#define MI_HOT_PARAMS                                                                                         \
+    const uint16_t* __restrict__ x, int hN0, int hnbatch, const uint8_t* __restrict__ hW0,                    \
+    const uint16_t* __restrict__ hsc0, const uint16_t* __restrict__ hnorm_w, const uint8_t* __restrict__ hW1, \
+    const uint16_t* __restrict__ hsc1, uint16_t* __restrict__ hy0
+#define MI_HOT_ARGS(x, L)                                                                                     \
+    (x), (L).s[0].N, (L).nbatch, (L).s[0].W, (L).s[0].sc, (L).norm_w, (L).nseg > 1 ? (L).s[1].W : nullptr,    \
+    (L).nseg > 1 ? (L).s[1].sc : nullptr, (L).s[0].y
+
 // ---- K known at compile time: x lives in registers ---------------------------------
 //
 // PIPE: each wavefront walks several row batches and keeps the next one in flight while it
@@ -229,7 +245,7 @@ __device__ __forceinline__ Seg find_segment(const SegList& L, int rb) {
 // RB row batches are fetched together, so that narrow rows (Q4, small K) still keep enough
 // bytes in flight per wavefront.
 template <int KIND, int KT, int VL, int EPI, bool PIPE, int RB, bool AM = false>
-__global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restrict__ x, const SegList L) {
+__global__ __launch_bounds__(kBlock) void gemv_fixed_k(MI_HOT_PARAMS, const SegList L) {
     using T = WT<KIND>;
     constexpr int LPR = kWave / VL, RPW = VL;
     constexpr int EIT = kWave * T::EPV;                 // elements per K-iteration
@@ -262,7 +278,14 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     const uint32_t lane_w = r * ROWB + koff / T::EPV * T::BPV;     // byte offset of the lane's weights
     const uint32_t lane_w0 = koff / T::EPV * T::BPV;               // same column, first row of the batch
     auto fetch = [&](Batch& b, int rb) {
-        const Seg sg = L.nseg == 1 ? L.s[0] : find_segment(L, rb);
+        // (one segment, or the two of a SwiGLU launch, whose second starts at batch hnbatch: all from the
+        //  arguments that came in registers; more segments: from the list)
+        Seg sg{hW0, hsc0, hy0, hN0, 0};
+        if constexpr (EPI == EPI_SWIGLU) {
+            if (rb >= hnbatch) sg = Seg{hW1, hsc1, hy0, hN0, hnbatch};
+        } else if (hW1 != nullptr) {
+            sg = find_segment(L, rb);
+        }
         const int row0 = (rb - sg.first) * RPW;
         const bool valid = row0 + r < sg.N;
         const int rr = valid ? r : 0;
@@ -272,7 +295,6 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
         b.yoff = valid ? r : -1;
         b.row0 = row0;
         if constexpr (KIND == WK_I8) b.s[0] = (sg.sc + row0)[rr];
-        if constexpr (EPI == EPI_ADD) b.res = b.ybase[rr];
         #pragma unroll
         for (int j = 0; j < NIT; ++j) {
             // lanes idle in a partial last iteration re-read the start of their row, so that
@@ -282,13 +304,15 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
             if constexpr (KIND == WK_Q4)
                 b.s[j] = (sg.sc + static_cast<size_t>(row0) * (KT / 32))[rr * (KT / 32) + (active ? j * 16 + (g * VL) / 4 : 0)];
         }
+        // (last: y's address is the one argument that does not come in registers)
+        if constexpr (EPI == EPI_ADD) b.res = b.ybase[rr];
     };
     const int nw = gridDim.x * kWavesPerBlock;
     int rb = blockIdx.x * kWavesPerBlock + wave;
     const int wid = rb;
     const TieRule rule{L.am_chunk};
     Cand top{kArgmaxNone, 0};                                 // AM: best row so far (lanes with g == 0)
-    if (rb >= L.nbatch) {
+    if (rb >= hnbatch) {
         if constexpr (AM) {
             if (lane == 0) { L.am_v[wid] = kArgmaxNone; L.am_i[wid] = 0; }
         }
@@ -302,7 +326,7 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     // result is dropped), so every fetch issues the same loads.
     auto fetch_group = [&](Group& gr, int at) {
         #pragma unroll
-        for (int u = 0; u < GB; ++u) fetch(gr.b[u], at + u * nw < L.nbatch ? at + u * nw : first);
+        for (int u = 0; u < GB; ++u) fetch(gr.b[u], at + u * nw < hnbatch ? at + u * nw : first);
     };
     const int step = nw * GB;
     // x (and the norm weights) are requested first and the first weights right behind them,
@@ -322,10 +346,10 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     //  takes its own copy of x in the norm's layout: lane l, elements 4 l + 256 j)
     constexpr int NJ = T::EPV == 8 ? (KT + 255) / 256 : 1;
     [[maybe_unused]] uint32_t xsq[NJ][2];
-    if (L.norm_w) {
+    if (hnorm_w) {
         #pragma unroll
         for (int j = 0; j < NIT; ++j)
-            load_dwords<XD, false>(nrm[j], L.norm_w + (j * EIT + koff < KT ? j * EIT + koff : koff));
+            load_dwords<XD, false>(nrm[j], hnorm_w + (j * EIT + koff < KT ? j * EIT + koff : koff));
         if constexpr (T::EPV == 8) {
             #pragma unroll
             for (int j = 0; j < NJ; ++j) {
@@ -336,14 +360,14 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     }
     Group g0, g1;
     fetch_group(g0, rb);
-    if constexpr (EPI == EPI_SWIGLU) fetch(g1.b[0], rb + L.s[1].first);
+    if constexpr (EPI == EPI_SWIGLU) fetch(g1.b[0], rb + hnbatch);
 
     // RMSNorm of x in place of a kernel of its own (QW/kernels/rmsnorm.cl: 64 lanes, each summing
     // the squares of elements 4 lane + 256 j, the same tree as the GEMV's, then
     // fp16((x * inv) * w)): the virtual lanes of this kernel own exactly those elements, so every
     // wavefront repeats the sum in the reference's order while its first weights are in flight.
     {
-        if (L.norm_w) {
+        if (hnorm_w) {
             float total;
             if constexpr (T::EPV == 4) {
                 float part[VL];
@@ -427,9 +451,9 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
                 g0.b[0].ybase[g0.b[0].yoff] = f_h((gv * sig) * uv);
             }
             rb += nw;
-            if (rb >= L.nbatch) break;
+            if (rb >= hnbatch) break;
             fetch(g0.b[0], rb);
-            fetch(g1.b[0], rb + L.s[1].first);
+            fetch(g1.b[0], rb + hnbatch);
         }
         return;
     }
@@ -456,13 +480,13 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
     auto consume_group = [&](const Group& gr, int at) {
         #pragma unroll
         for (int u = 0; u < GB; ++u)
-            if (at + u * nw < L.nbatch) consume(gr.b[u]);
+            if (at + u * nw < hnbatch) consume(gr.b[u]);
     };
     if constexpr (!PIPE) {
         while (true) {
             consume_group(g0, rb);
             rb += step;
-            if (rb >= L.nbatch) break;
+            if (rb >= hnbatch) break;
             fetch_group(g0, rb);
         }
     } else {
@@ -470,11 +494,11 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
             fetch_group(g1, rb + step);
             consume_group(g0, rb);
             rb += step;
-            if (rb >= L.nbatch) break;
+            if (rb >= hnbatch) break;
             fetch_group(g0, rb + step);
             consume_group(g1, rb);
             rb += step;
-            if (rb >= L.nbatch) break;
+            if (rb >= hnbatch) break;
         }
     }
     if constexpr (AM) {
@@ -498,7 +522,7 @@ __global__ __launch_bounds__(kBlock) void gemv_fixed_k(const uint16_t* __restric
 // 16 lanes still share a row and a wavefront still streams row batches of 4 rows with the
 // same double-buffered fetch; each lane owns one scale block per K-iteration.
 template <int KT, int EPI, bool PIPE, int RB, bool AM = false>
-__global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restrict__ x, const SegList L) {
+__global__ __launch_bounds__(kBlock) void gemv_q4_fast(MI_HOT_PARAMS, const SegList L) {
     constexpr int EIT = 512;                            // elements per K-iteration (16 lanes x 32)
     constexpr int NIT = (KT + EIT - 1) / EIT;
     constexpr int ROWB = KT / 2;
@@ -521,7 +545,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
     };
     const uint32_t lane_w = r * ROWB + g * 16, lane_w0 = g * 16;
     auto fetch = [&](Batch& b, int rb) {
-        const Seg sg = L.nseg == 1 ? L.s[0] : find_segment(L, rb);
+        const Seg sg = hW1 == nullptr ? Seg{hW0, hsc0, hy0, hN0, 0} : find_segment(L, rb);
         const int row0 = (rb - sg.first) * 4;
         const bool valid = row0 + r < sg.N;
         const int rr = valid ? r : 0;
@@ -547,7 +571,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
     const int wid = rb;
     const TieRule rule{L.am_chunk};
     Cand top{kArgmaxNone, 0};                                 // AM: best row so far (lanes with g == 0)
-    if (rb >= L.nbatch) {
+    if (rb >= hnbatch) {
         if constexpr (AM) {
             if (lane == 0) { L.am_v[wid] = kArgmaxNone; L.am_i[wid] = 0; }
         }
@@ -567,7 +591,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
     const int first = rb;
     auto fetch_group = [&](Group& gr, int at) {
         #pragma unroll
-        for (int u = 0; u < GB; ++u) fetch(gr.b[u], at + u * nw < L.nbatch ? at + u * nw : first);
+        for (int u = 0; u < GB; ++u) fetch(gr.b[u], at + u * nw < hnbatch ? at + u * nw : first);
     };
     Group g0, g1;
     fetch_group(g0, rb);
@@ -632,14 +656,14 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
     auto consume_group = [&](const Group& gr, int at) {
         #pragma unroll
         for (int u = 0; u < GB; ++u)
-            if (at + u * nw < L.nbatch) consume(gr.b[u]);
+            if (at + u * nw < hnbatch) consume(gr.b[u]);
     };
     const int step = nw * GB;
     if constexpr (!PIPE) {
         while (true) {
             consume_group(g0, rb);
             rb += step;
-            if (rb >= L.nbatch) break;
+            if (rb >= hnbatch) break;
             fetch_group(g0, rb);
         }
     } else {
@@ -647,11 +671,11 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
             fetch_group(g1, rb + step);
             consume_group(g0, rb);
             rb += step;
-            if (rb >= L.nbatch) break;
+            if (rb >= hnbatch) break;
             fetch_group(g0, rb + step);
             consume_group(g1, rb);
             rb += step;
-            if (rb >= L.nbatch) break;
+            if (rb >= hnbatch) break;
         }
     }
     if constexpr (AM) {
@@ -662,7 +686,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(const uint16_t* __restric
 
 // ---- K known at run time: x is staged once per block in LDS ------------------------
 template <int KIND, int VL, int EPI>
-__global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict__ x, const SegList L, int K) {
+__global__ __launch_bounds__(kBlock) void gemv_any_k(MI_HOT_PARAMS, const SegList L, int K) {
     using T = WT<KIND>;
     constexpr int LPR = kWave / VL, RPW = VL;
     constexpr int EIT = kWave * T::EPV;
@@ -685,8 +709,8 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(const uint16_t* __restrict_
     const size_t rowb = static_cast<size_t>(K) / T::EPV * T::BPV;
     const int nit = (K + EIT - 1) / EIT;
 
-    for (int rb = blockIdx.x * kWavesPerBlock + wave; rb < L.nbatch; rb += gridDim.x * kWavesPerBlock) {
-        const Seg sg = find_segment(L, rb);
+    for (int rb = blockIdx.x * kWavesPerBlock + wave; rb < hnbatch; rb += gridDim.x * kWavesPerBlock) {
+        const Seg sg = hW1 == nullptr ? Seg{hW0, hsc0, hy0, hN0, 0} : find_segment(L, rb);
         const int row = (rb - sg.first) * RPW + r;
         const bool valid = row < sg.N;
         const int rowc = valid ? row : sg.N - 1;
@@ -949,9 +973,9 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
     case KT:                                                                                             \
         if (PIPE_OK && p.pipe) {                                                                         \
             constexpr int kRB = group_size(KIND, KT, VL);                                                \
-            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, PIPE_OK, kRB>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, PIPE_OK, kRB>), p.grid, dim3(kBlock), 0, s, MI_HOT_ARGS(x, p.L), p.L); \
         } else {                                                                                         \
-            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, false, 1>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, false, 1>), p.grid, dim3(kBlock), 0, s, MI_HOT_ARGS(x, p.L), p.L); \
         }                                                                                                \
         break;
     if constexpr (EPI == EPI_STORE && KIND != WK_Q4) {
@@ -960,9 +984,9 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
     case KT:                                                                                             \
         if (PIPE_OK && p.pipe) {                                                                         \
             constexpr int kRB = group_size(KIND, KT, VL);                                                \
-            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, PIPE_OK, kRB, true>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, PIPE_OK, kRB, true>), p.grid, dim3(kBlock), 0, s, MI_HOT_ARGS(x, p.L), p.L); \
         } else {                                                                                         \
-            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, false, 1, true>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+            hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI, false, 1, true>), p.grid, dim3(kBlock), 0, s, MI_HOT_ARGS(x, p.L), p.L); \
         }                                                                                                \
         break;
             switch (K) {
@@ -987,7 +1011,7 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
         MI_FIXED(4864, false)
         default: {
             const size_t lds = static_cast<size_t>(K) * 2;
-            hipLaunchKernelGGL((gemv_any_k<KIND, VL, EPI>), p.grid, dim3(kBlock), lds, s, x, p.L, K);
+            hipLaunchKernelGGL((gemv_any_k<KIND, VL, EPI>), p.grid, dim3(kBlock), lds, s, MI_HOT_ARGS(x, p.L), p.L, K);
         }
     }
 #undef MI_FIXED
@@ -1006,7 +1030,7 @@ bool launch_swiglu_vl(hipStream_t s, const GemvCall* calls) {
     p.grid = dim3((waves + kWavesPerBlock - 1) / kWavesPerBlock, 1, 1);
     const auto* x = static_cast<const uint16_t*>(calls[0].x);
 #define MI_SWIGLU(KT) \
-    case KT: hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI_SWIGLU, false, 1>), p.grid, dim3(kBlock), 0, s, x, p.L); break;
+    case KT: hipLaunchKernelGGL((gemv_fixed_k<KIND, KT, VL, EPI_SWIGLU, false, 1>), p.grid, dim3(kBlock), 0, s, MI_HOT_ARGS(x, p.L), p.L); break;
     switch (calls[0].K) {
         MI_SWIGLU(576)
         MI_SWIGLU(896)
@@ -1030,9 +1054,9 @@ bool launch_q4_fast(hipStream_t s, const GemvCall* calls, int n, bool* taken) {
     case KT:                                                                                         \
         if (p.pipe) {                                                                                \
             constexpr int kRB = group_size(WK_Q4, KT, 4);                                            \
-            hipLaunchKernelGGL((gemv_q4_fast<KT, EPI, true, kRB, AM>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+            hipLaunchKernelGGL((gemv_q4_fast<KT, EPI, true, kRB, AM>), p.grid, dim3(kBlock), 0, s, MI_HOT_ARGS(x, p.L), p.L); \
         } else {                                                                                     \
-            hipLaunchKernelGGL((gemv_q4_fast<KT, EPI, false, 1, AM>), p.grid, dim3(kBlock), 0, s, x, p.L); \
+            hipLaunchKernelGGL((gemv_q4_fast<KT, EPI, false, 1, AM>), p.grid, dim3(kBlock), 0, s, MI_HOT_ARGS(x, p.L), p.L); \
         }                                                                                            \
         break;
     if constexpr (EPI == EPI_STORE) {
