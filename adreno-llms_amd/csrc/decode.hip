@@ -274,15 +274,16 @@ constexpr int kTileRows = 128;
 constexpr int kMaxPositions = 8192;                      // longest context a decoder is created for
 
 template <int D>
-__global__ __launch_bounds__(256) void rope_attention_tiled(const uint16_t* __restrict__ q_raw, const uint16_t* __restrict__ k_raw,
+// (Arguments in the order of need: the first 14 dwords arrive in registers with the wavefront, and the
+//  first thing the kernel does is ask for the cache tiles and the position.)
+__global__ __launch_bounds__(256) void rope_attention_tiled(uint16_t* __restrict__ kc, uint16_t* __restrict__ vc,
+                                      const State* __restrict__ st, int n_heads, int n_kv_heads, int max_pos,
+                                      float scale, const uint16_t* __restrict__ q_raw, const uint16_t* __restrict__ k_raw,
                                       const uint16_t* __restrict__ v_raw, const uint16_t* __restrict__ bq,
                                       const uint16_t* __restrict__ bk, const uint16_t* __restrict__ bv,
                                       const uint16_t* __restrict__ rope_now,
-                                      uint16_t* __restrict__ kc, uint16_t* __restrict__ vc,
                                       uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_out,
-                                      uint16_t* __restrict__ v_out, uint16_t* __restrict__ out,
-                                      const State* __restrict__ st, int n_heads, int n_kv_heads, int max_pos,
-                                      float scale) {
+                                      uint16_t* __restrict__ v_out, uint16_t* __restrict__ out) {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     constexpr int kRowH = D + 8;                           // tile row stride in halves
     constexpr int kPieces = D / 8;                         // 16-byte pieces per row
@@ -1191,13 +1192,13 @@ int mi_decoder_step(void* dec, void* stream) {
         if (D == 64 || D == 128) {
             const size_t lds = tiled_attention_lds(D, c.max_pos);
             if (D == 64)
-                hipLaunchKernelGGL(rope_attention_tiled<64>, dim3(c.n_heads), dim3(256), lds, s, d->q, d->k, d->v, bq, bk, bv,
-                                   d->rope_now, kc, vc, d->qr, d->kr, d->vr, d->attn, d->st, c.n_heads, c.n_kv_heads,
-                                   c.max_pos, scale);
+                hipLaunchKernelGGL(rope_attention_tiled<64>, dim3(c.n_heads), dim3(256), lds, s, kc, vc, d->st, c.n_heads,
+                                   c.n_kv_heads, c.max_pos, scale, d->q, d->k, d->v, bq, bk, bv, d->rope_now, d->qr, d->kr,
+                                   d->vr, d->attn);
             else
-                hipLaunchKernelGGL(rope_attention_tiled<128>, dim3(c.n_heads), dim3(256), lds, s, d->q, d->k, d->v, bq, bk, bv,
-                                   d->rope_now, kc, vc, d->qr, d->kr, d->vr, d->attn, d->st, c.n_heads, c.n_kv_heads,
-                                   c.max_pos, scale);
+                hipLaunchKernelGGL(rope_attention_tiled<128>, dim3(c.n_heads), dim3(256), lds, s, kc, vc, d->st, c.n_heads,
+                                   c.n_kv_heads, c.max_pos, scale, d->q, d->k, d->v, bq, bk, bv, d->rope_now, d->qr, d->kr,
+                                   d->vr, d->attn);
         } else {
             // a whole number of wavefronts: the maximum's cross-lane steps read every lane of a wavefront
             const int at = ((D > 64 ? D : 64) + 63) & ~63;
