@@ -1397,8 +1397,9 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
         case 2: return launch_tile<64, 64, 32, 32>(s, kind, M, N, K, x, W, scale, out);
         case 3: return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);
         default:
-            MI_ERROR_FMT("gemm: mode %d has no kernel for kind=%d M=%d N=%d K=%d (Q4 weights take the wide kernel "
-                         "only; its 32-bit offsets reach 4 GiB of x and of W)", gemm_mode(s), static_cast<int>(kind), M, N, K);
+            MI_ERROR_FMT("gemm: mode %d has no kernel for kind=%d M=%d N=%d K=%d (Q4 weights have no tile kernel; the "
+                         "streaming kernel takes up to 64 rows of x; the wide kernel's 32-bit offsets reach 4 GiB of x and "
+                         "of W)", gemm_mode(s), static_cast<int>(kind), M, N, K);
             return false;
     }
 }
