@@ -901,7 +901,15 @@ inline int resident_waves() { return device_info().cus * 3 * kWavesPerBlock; }
 // VL virtual lanes are whole in the K tail.
 int pick_vl(WeightKind kind, int M, long rows, int K) {
     const int epv = kind == WK_Q4 ? 8 : 4;
-    const int max_vl = kind == WK_F16 ? 2 : 4;
+    int max_vl = kind == WK_F16 ? 2 : 4;
+    // The kernels that hold x in registers spend K VL / 128 of them on it: at a long K the wide
+    // tiles run short (K = 4864 with four rows per lane spills) and stream at half the rate of the
+    // one-row tile.  Cold, 16 384 rows, four / two / one row per lane, us: int8 K = 4864 31.0 / 23.1 /
+    // 15.0, K = 4608 25.6 / 22.0 / 14.4, K = 2560 11.3 / 9.8 / 9.6; Q4 K = 4608 17.0 / 13.5 / 11.6, K = 2560
+    // 7.6 / 7.8 / 8.2; fp16 K = 4864 - / 28.8 / 27.2.  (The kernel with x in LDS, for every other long K,
+    // keeps the wide tile: int8 16 384 x 4096 in 18.8 / 19.3 / 25.3 us.)
+    if (K == 4608 || K == 4864) max_vl = 1;
+    else if (K == 2560 && kind != WK_Q4) max_vl = 2;
     const long waves_wanted = 4L * device_info().cus;
     int narrowest = 1;
     for (int vl = max_vl; vl >= 1; vl >>= 1) {
