@@ -684,6 +684,24 @@ __global__ __launch_bounds__(kBlock) void gemv_q4_fast(MI_HOT_PARAMS, const SegL
     }
 }
 
+// x (K halves, K % 4 == 0, 8-byte aligned) into LDS by the whole block.  Where K is long a thread
+// requests four 8-byte pieces before it stores the first (one trip to memory per 4096 halves instead
+// of one per 512); what is left goes piece by piece.
+__device__ __forceinline__ void stage_x(uint32_t* xs, const uint16_t* x, int K) {
+    const uint2* src = reinterpret_cast<const uint2*>(x);
+    uint2* dst = reinterpret_cast<uint2*>(xs);
+    const int n = K / 4;
+    int base = 0;
+    for (; base + 4 * kBlock <= n; base += 4 * kBlock) {
+        uint2 t[4];
+        #pragma unroll
+        for (int u = 0; u < 4; ++u) t[u] = src[base + u * kBlock + static_cast<int>(threadIdx.x)];
+        #pragma unroll
+        for (int u = 0; u < 4; ++u) dst[base + u * kBlock + static_cast<int>(threadIdx.x)] = t[u];
+    }
+    for (int i = 2 * base + static_cast<int>(threadIdx.x); i < K / 2; i += kBlock) xs[i] = reinterpret_cast<const uint32_t*>(x)[i];
+}
+
 // ---- K known at run time: x is staged once per block in LDS ------------------------
 template <int KIND, int VL, int EPI>
 __global__ __launch_bounds__(kBlock) void gemv_any_k(MI_HOT_PARAMS, const SegList L, int K) {
@@ -698,7 +716,7 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(MI_HOT_PARAMS, const SegLis
 
     const int m = blockIdx.y;
     x += static_cast<size_t>(m) * K;
-    for (int i = threadIdx.x; i < K / 2; i += kBlock) xs[i] = reinterpret_cast<const uint32_t*>(x)[i];
+    stage_x(xs, x, K);
     __syncthreads();
 
     const int lane = threadIdx.x % kWave;
@@ -798,7 +816,7 @@ __global__ __launch_bounds__(kBlock) void gate_up_silu_any_k(const uint16_t* __r
     constexpr int ITB = kWave * T::BPV;
     constexpr int kChunk = 2;                           // K-iterations of each matrix per register buffer (4 and 8 measured no better)
     extern __shared__ uint32_t xs[];
-    for (int i = threadIdx.x; i < K / 2; i += kBlock) xs[i] = reinterpret_cast<const uint32_t*>(x)[i];
+    stage_x(xs, x, K);
     __syncthreads();
 
     const int lane = threadIdx.x % kWave;

@@ -216,7 +216,7 @@ def test_silu_gate_epilogue(queue, kind, N, K):
 
 
 @pytest.mark.parametrize("kind", ["i8", "f16"])
-@pytest.mark.parametrize("N,K", [(1536, 576), (4864, 896), (50, 64)])
+@pytest.mark.parametrize("N,K", [(1536, 576), (4864, 896), (50, 64), (130, 4104)])
 def test_gate_up_silu_epilogue(queue, kind, N, K):
     Wg, Wu, x = synth_w(18, N, K), synth_w(19, N, K), synth_x(20, K)
     xb, ob = mil.Buffer.from_host(x), mil.Buffer(N * 2)
