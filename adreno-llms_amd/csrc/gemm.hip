@@ -896,12 +896,25 @@ __global__ __launch_bounds__(64 * kWaves) void gemm_skinny(const uint16_t* __res
     const int it0 = b0 + (b1 - b0) * slice / ks, it1 = b0 + (b1 - b0) * (slice + 1) / ks;
 
     if constexpr (XL) {
+        // Wavefront w copies rows w, w + 8, ...: a lane requests its 16-byte piece of each of the wavefront's
+        // 2 MT rows before it stores the first, so the copy is one trip to memory per 64 pieces of a row
+        // (before: a trip per 512 pieces of the tile, and a division per piece; 4864 x 896 at 16 / 32 / 48
+        // rows 4.65 / 5.8 / 6.8 -> 4.35 / 4.95 / 5.7 us).  Rows past M are read as the last row and never
+        // stored from.  Asking for the first weights ahead of this copy was measured as well: slower
+        // (4.7 / 5.4 / 6.05 us), x then arrives behind them.
         const int per_row = K / 8;                       // 16-byte pieces per row
-        for (int idx = threadIdx.x; idx < 16 * MT * per_row; idx += 64 * kWaves) {
-            const int row = idx / per_row, piece = idx - row * per_row;
-            const int m = row < M ? row : M - 1;         // rows past M are read as the last row (and never stored)
-            *reinterpret_cast<u32x4*>(lds + row * xrow + piece * 16) =
-                *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint8_t*>(X) + static_cast<size_t>(m) * K * 2 + piece * 16);
+        const uint8_t* Xb = reinterpret_cast<const uint8_t*>(X);
+        for (int piece = threadIdx.x & 63; piece < per_row; piece += 64) {
+            u32x4 t[2 * MT];
+            #pragma unroll
+            for (int rr = 0; rr < 2 * MT; ++rr) {
+                const int row = wave + kWaves * rr;
+                const int m = row < M ? row : M - 1;
+                t[rr] = *reinterpret_cast<const u32x4*>(Xb + static_cast<size_t>(m) * K * 2 + piece * 16);
+            }
+            #pragma unroll
+            for (int rr = 0; rr < 2 * MT; ++rr)
+                *reinterpret_cast<u32x4*>(lds + (wave + kWaves * rr) * xrow + piece * 16) = t[rr];
         }
         __syncthreads();
     }
@@ -1152,22 +1165,30 @@ inline Shape pick_shape(int kind, int M, int N, int K, int cus, size_t workspace
     return sh;
 }
 
-// Where the streaming kernel is the library's own choice (measured against the tiles above, int8,
-// warm weights, us).  With x in LDS, or one strip per block: up to 48 rows (4864 x 896: 4.9 / 6.0 /
-// 7.0 at 16 / 32 / 48 rows against 8.0 for the 64 x 64 tiles, 8.4 against 7.4 at 64; 2560 x 1024: 4.4 /
-// 5.3 / 6.7 against 9.2 / 9.3 / 8.9, 7.7 against 7.3 at 64); up to 64 rows where K is cut over blocks
-// as well (896 x 4864: 7.1 / 8.3 / 10.8 at 16 / 32 / 64 rows against 12.1 / 11.0 / 11.9; 1024 x 4608: 7.3 /
-// 8.5 / 10.9 against 10 to 11.4).  With x from the caches and shared by several strips per block,
-// only up to 16 rows (8192 x 2048 at 48 rows: 28 us against 17).  And no more strips than stay
-// resident at once: an lm_head of 151 936 rows streams at 4.0 TB/s here (a wavefront loads a
-// strip, waits, multiplies) against 4.8 TB/s in the wide kernel.
+// Where the streaming kernel is the library's own choice (measured against the tiles above, warm
+// weights, us).
+//  - With x in LDS, or one strip per block: up to 48 rows (int8 4864 x 896: 4.4 / 5.0 / 5.7 at 16 / 32 / 48
+//    rows against 6.3 to 6.5 for the 64 x 64 tiles, 6.65 against 6.5 at 64; 2560 x 1024: 4.4 / 5.4 / 6.5
+//    against 8.2 to 9.1); up to 64 where K is cut over blocks as well (896 x 4864: 6.9 / 8.0 / 10.5 at 16 /
+//    32 / 64 rows against 25 and more unsliced, 12 to 14 as the wide kernel was chosen in slices).
+//  - x in LDS, Q4 or fp16 weights of a few MB: up to 64 rows (Q4 4864 x 896 at 64 rows 8.55 against
+//    11.8 for the wide kernel, 9728 x 896 10.5 against 12.4; fp16 4864 x 896 7.5 against 8.0).
+//  - x from the caches and shared by several strips per block: only up to 16 rows (8192 x 2048 at 48
+//    rows: 28 us against 17).  Q4 then holds twice the x per iteration in registers: one strip per
+//    block is good for 48 rows (2560 x 1024: 7.5 against 10.7, 3072 x 1024: 7.6 against 10.9), K over
+//    blocks as well for 32 (896 x 4864: 10.3 / 14.0 / 26.5 at 32 / 48 / 64 rows against 12.7 to 12.9).
+//  - No more than 13.5 MB of weights: beyond that the launch is long enough for the wide kernel's
+//    higher streaming rate to win (a wavefront here loads a strip, waits, multiplies).  int8 14 592 x
+//    896 (13.1 MB) 6.4 / 7.0 / 7.9 at 16 / 32 / 48 rows against 8.5, but 19 456 x 896 8.8 / 9.6 / 10.5 against
+//    8.6 / 8.7 / 9.0, 49 152 x 576 11.2 against 7.3 and fp16 49 152 x 576 16.7 against 10.8; an lm_head of
+//    151 936 rows streams at 4.0 TB/s here against 4.8 TB/s there.
 inline bool preferred(int kind, int M, int N, int K, int cus, size_t workspace_bytes) {
     const Shape sh = pick_shape(kind, M, N, K, cus, workspace_bytes);
+    const double w_bytes = static_cast<double>(N) * K * (kind == WK_F16 ? 2.0 : kind == WK_Q4 ? 0.5625 : 1.0);
     int rows = sh.xl || sh.ks == kWaves ? (sh.kb > 1 ? 64 : 48) : 16;
-    // Q4 with x from the caches holds twice the x per iteration in registers: 48 rows spill a little,
-    // 64 a lot (896 x 4864: 10.5 / 13.7 / 26.8 us at 32 / 48 / 64 rows)
-    if (kind == WK_Q4 && !sh.xl && rows > 32) rows = 32;
-    return M <= rows && (N + 15) / 16 <= 16L * cus;
+    if (kind == WK_Q4 && !sh.xl) rows = sh.ks == kWaves && sh.kb == 1 ? 48 : rows > 32 ? 32 : rows;
+    if (kind != WK_I8 && sh.xl && w_bytes <= (kind == WK_Q4 ? 6.0e6 : 9.0e6)) rows = 64;
+    return M <= rows && w_bytes <= 13.5e6 && (N + 15) / 16 <= 16L * cus;
 }
 
 // Estimated time (us), fitted to the same measurements.

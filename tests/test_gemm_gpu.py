@@ -218,6 +218,19 @@ def test_streaming_gemm_is_the_choice_for_a_few_rows_and_refuses_more_than_64(qu
         mil.nnopt_unregister_weight(wb)
 
 
+def test_streaming_gemm_is_not_the_choice_for_many_megabytes_of_weights(queue):
+    """A long launch belongs to the wide kernel, which streams faster: an lm_head of 49 152 x 576 (28 MB
+    of int8) at 16 rows of x takes the wide kernel, 14 592 x 896 (13 MB) still streams.  Plans only."""
+    for (N, K, kernel) in ((49152, 576, 1), (14592, 896, 4)):
+        wb, sb = mil.Buffer(N * K), mil.Buffer(N * 2)
+        xb = mil.Buffer(16 * K * 2)
+        assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+        try:
+            assert mil.linear_plan(queue, 16, N, K, xb, wb)[0] == kernel, (N, K, mil.linear_plan(queue, 16, N, K, xb, wb))
+        finally:
+            mil.nnopt_unregister_weight(wb)
+
+
 @pytest.mark.parametrize("kind", ["i8", "f16", "q4", "q4_single_rounding"])
 def test_streaming_gemm_exact_on_integer_data_and_indices(queue, kind):
     """Small integers: every sum is exact whatever the order, so the result is integer arithmetic's
