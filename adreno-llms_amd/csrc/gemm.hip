@@ -790,7 +790,13 @@ inline double estimate_us(int kind, int terms, int tm, int splits, int M, int N,
     const double block_us = (2.6 + 0.5 * tm + stages * stage_us) * (per_cu == 2 ? 1.4 : 1.0);
     const long slots = static_cast<long>(cus) * per_cu;
     const long full = blocks / slots, rem = blocks % slots;
-    double t = full * 1.56 * block_us + (rem ? (1.0 + 0.56 * rem / slots) * block_us : 0.0);
+    // (64-row tiles of int8 / fp16 weights, unsliced, on more than half of the CUs and at most one per CU,
+    //  run nearly as on an empty chip: 512 x 4864 x 896 in 11.2 us where the general factor says 13.6 and the
+    //  64 x 64 tiles, estimated at 13.5, take 13.2; 2048 x 1152 x 896 13.2 against 15.9, 512 x 4608 x 1024 12.1
+    //  against 14.5, 4096 x 576 x 1536 18.9 against 33.5.  With fewer blocks the long serial K of such
+    //  shapes decides and the general factor holds: 2048 x 896 x 4864 unsliced 47 against 37 us in two slices.)
+    const double crowd = tm == 2 && splits == 1 && kind != WK_Q4 && blocks > cus / 2 && blocks <= cus ? 0.2 : 0.56;
+    double t = full * 1.56 * block_us + (rem ? (1.0 + crowd * rem / slots) * block_us : 0.0);
     // every row of tiles streams W again: not faster than that many bytes at about 6.4 TB/s, or,
     // for a W that stays in the memory-side cache (32 MB taken as the limit), 2.2 times that for
     // the reads after the first
