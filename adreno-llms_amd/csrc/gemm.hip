@@ -789,13 +789,19 @@ inline double estimate_us(int kind, int terms, int tm, int splits, int M, int N,
     const int per_cu = blocks > cus ? blocks_per_cu(kind, tm) : 1;
     const double block_us = (2.6 + 0.5 * tm + stages * stage_us) * (per_cu == 2 ? 1.4 : 1.0);
     const long slots = static_cast<long>(cus) * per_cu;
-    const long full = blocks / slots, rem = blocks % slots;
+    const long full = (blocks - 1) / slots, rem = blocks - full * slots;     // the last round, full or not, is `rem`
     // (64-row tiles of int8 / fp16 weights, unsliced, on more than half of the CUs and at most one per CU,
     //  run nearly as on an empty chip: 512 x 4864 x 896 in 11.2 us where the general factor says 13.6 and the
     //  64 x 64 tiles, estimated at 13.5, take 13.2; 2048 x 1152 x 896 13.2 against 15.9, 512 x 4608 x 1024 12.1
     //  against 14.5, 4096 x 576 x 1536 18.9 against 33.5.  With fewer blocks the long serial K of such
-    //  shapes decides and the general factor holds: 2048 x 896 x 4864 unsliced 47 against 37 us in two slices.)
-    const double crowd = tm == 2 && splits == 1 && kind != WK_Q4 && blocks > cus / 2 && blocks <= cus ? 0.2 : 0.56;
+    //  shapes decides and the general factor holds: 2048 x 896 x 4864 unsliced 47 against 37 us in two slices.
+    //  32-row tiles likewise at a K of 1280 to 3072, where the 64 x 64 tiles slow down as soon as a CU holds
+    //  two of them: 1536 x 576 x 1536 19.2 -> 14.6 us, 1024 x 2048 x 2048 23.2 -> 18.4, 192 x 8192 x 2048 21.6 ->
+    //  17.3, fp16 1536 x 1024 x 2560 29.6 -> 22.7; at a shorter K the 64 x 64 tiles stay ahead (1536 x 1152 x 896
+    //  10.2 against 11.2), at a longer one slices do (1536 x 896 x 4864 32.6 against 37.7).)
+    const bool roomy = splits == 1 && kind != WK_Q4 && blocks > cus / 2 && blocks <= cus &&
+                       (tm == 2 || (tm == 1 && stages >= 20 && stages <= 48));
+    const double crowd = roomy ? 0.2 : 0.56;
     double t = full * 1.56 * block_us + (rem ? (1.0 + crowd * rem / slots) * block_us : 0.0);
     // every row of tiles streams W again: not faster than that many bytes at about 6.4 TB/s, or,
     // for a W that stays in the memory-side cache (32 MB taken as the limit), 2.2 times that for
@@ -1321,7 +1327,11 @@ double tiled_estimate_us(int M, int N, int K) {
     const int nk = K / kKT;
     const long t64 = tiles(M, N, 64, 64);
     const double serial = (0.9 + nk * 0.4) * (1.0 + 0.3 * (t64 < 128 ? t64 / 128.0 : 1.0));
-    const double bulk = 3.3 + t64 * nk * (nk > 32 ? 0.00155 : 0.0012);
+    // (at a long K the CUs that hold a second tile set the time: 192 x 8192 x 2048, 384 tiles, takes the
+    //  22 us of 512 tiles; whole rounds of CUs then)
+    const int cus = device_info().cus;
+    const long counted = nk >= 20 && t64 > cus ? (t64 + cus - 1) / cus * cus : t64;
+    const double bulk = 3.3 + counted * nk * (nk > 32 ? 0.00155 : 0.0012);
     return serial > bulk ? serial : bulk;
 }
 
