@@ -1207,7 +1207,12 @@ inline bool preferred(int kind, int M, int N, int K, int cus, size_t workspace_b
 inline double estimate_us(int kind, int M, int N, int K, int cus, size_t workspace_bytes) {
     const Shape sh = pick_shape(kind, M, N, K, cus, workspace_bytes);
     const double w_bytes = static_cast<double>(N) * K * (kind == WK_F16 ? 2.0 : kind == WK_Q4 ? 0.5625 : 1.0);
-    return sh.xl ? 3.75 + 0.035 * M + w_bytes / 8.0e6 : (sh.kb > 1 ? 5.4 : 3.6) + 0.07 * M + w_bytes / 8.0e6;
+    // (Q4 weights: the two-term feed costs 0.6 us more, 1.1 with K over blocks)
+    const double q4_us = kind == WK_Q4 ? (sh.kb > 1 ? 1.1 : 0.6) : 0.0;
+    // (x from the caches: 0.07 us per row where several strips of a block read it, 0.03 where the block's
+    //  eight wavefronts share one strip, 0.06 with K over blocks as well)
+    const double xg_us = sh.kb > 1 ? 5.4 + 0.06 * M : sh.ks == kWaves ? 3.6 + 0.03 * M : 3.6 + 0.07 * M;
+    return q4_us + (sh.xl ? 3.75 + 0.035 * M : xg_us) + w_bytes / 8.0e6;
 }
 
 template <int KIND, int MT, int SW, bool XL, int TERMS>

@@ -338,16 +338,20 @@ int mi_stream_set_modes(void* stream, int gemv_mode, int gemm_mode) {
 
 // M > 1: a real contraction goes to the MFMA GEMM.  Every batch in mode 1, and shapes the GEMM
 // does not take, run the GEMV once per row of x, as the reference's quantised prefill does; so
-// do batches below 16 rows while that is estimated to be faster (each GEMV row streams W again:
-// about 0.25 us + bytes / 6.6 TB/s per row; measured int8, warm: 1536 x 576 2.95 us for two rows,
-// 4864 x 896 3.8 / 5.0 us and 896 x 4864 3.85 / 6.15 us for two / four).
+// do batches below 16 rows while that is estimated to be faster.  The rows of one launch run side by
+// side and all but the first find W in the caches: measured under graph replay, every kind of
+// weights, 2.45 us + 0.15 us per row and million weights (int8 1152 x 896: 2.7 / 3.2 / 3.7 us for 2 / 4 / 8
+// rows, 4864 x 896: 3.7 / 4.8 / 7.4 us, 9728 x 896: 5.6 / 8.5 / 13.6 us; fp16 and Q4 within a tenth of
+// that), against 3.8 to 4.6 us for the GEMM of a small matrix whatever its rows.
 static bool takes_gemm(hipStream_t s, const Entry& e, int M, int N, int K, const void* x, const void* W) {
     const int mode = gemm_mode(s);
     if (M < 2 || mode == 1 || !gemm_supported(e.kind, M, N, K, x, W, e.scale)) return false;
     if (M >= 16 || mode != 0) return true;
-    const double w_bytes = static_cast<double>(N) * K * (e.kind == WK_F16 ? 2.0 : e.kind == WK_I8 ? 1.0 : 0.5625);
-    const double row_us = 0.25 + w_bytes / 6.6e6;
-    return gemm_estimate_us(e.kind, M, N, K, workspace_of(s) ? kWorkspaceBytes : 0) < 2.4 + M * row_us;
+    // (fp16 rows cost 1.15 times that, 1.8 times at a K of 4096 and more, where a lane holds one row;
+    //  Q4 rows 0.05 us more)
+    const double kind_factor = e.kind == WK_F16 ? (K >= 4096 ? 1.8 : 1.15) : 1.0;
+    const double row_us = 0.02 + (e.kind == WK_Q4 ? 0.05 : 0.0) + kind_factor * 0.15e-6 * static_cast<double>(N) * K;
+    return gemm_estimate_us(e.kind, M, N, K, workspace_of(s) ? kWorkspaceBytes : 0) < 2.45 + M * row_us;
 }
 
 int mi_linear(void* stream, int M, int N, int K, const void* x, const void* W, void* out) {
