@@ -803,13 +803,13 @@ inline double estimate_us(int kind, int terms, int tm, int splits, int M, int N,
                        (tm == 2 || (tm == 1 && stages >= 20 && stages <= 48));
     const double crowd = roomy ? 0.2 : 0.56;
     double t = full * 1.56 * block_us + (rem ? (1.0 + crowd * rem / slots) * block_us : 0.0);
-    // every row of tiles streams W again: not faster than that many bytes at about 6.4 TB/s, or,
+    // every row of tiles streams W again: not faster than that many bytes at about 6.8 TB/s, or,
     // for a W that stays in the memory-side cache (32 MB taken as the limit), 2.2 times that for
     // the reads after the first
     const double w_once = static_cast<double>(N) * K * (kind == WK_F16 ? 2.0 : kind == WK_I8 ? 1.0 : 0.5625);
     const int tiles_m = (M + 32 * tm - 1) / (32 * tm);
     const double w_bytes = w_once <= 32.0e6 ? w_once * (1.0 + (tiles_m - 1) / 2.2) : w_once * tiles_m;
-    if (t < 2.5 + w_bytes / 6.4e6) t = 2.5 + w_bytes / 6.4e6;
+    if (t < 2.5 + w_bytes / 6.8e6) t = 2.5 + w_bytes / 6.8e6;
     if (splits > 1) t += 2.5 + 2.0 * splits * M * static_cast<double>(N) * 4 / 4.0e6;   // ~4 TB/s there and back
     return t;
 }
@@ -821,6 +821,7 @@ inline void pick_shape(int kind, int terms, int M, int N, int K, int cus, size_t
     static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24};
     double best_t = 1e30;
     for (int tm = 1; tm <= 5; ++tm) {
+        if (32 * (tm - 1) >= M) break;                   // no tile taller than x needs (16 x 49 152 x 576: 7.8 against 8.7 us)
         for (int sp : kSplits) {
             if (sp > 1 && (K / 64 < 2 * sp || static_cast<double>(sp) * M * N * 4 > static_cast<double>(workspace_bytes)))
                 continue;
@@ -1332,10 +1333,12 @@ double tiled_estimate_us(int M, int N, int K) {
     const int nk = K / kKT;
     const long t64 = tiles(M, N, 64, 64);
     const double serial = (0.9 + nk * 0.4) * (1.0 + 0.3 * (t64 < 128 ? t64 / 128.0 : 1.0));
-    // (at a long K the CUs that hold a second tile set the time: 192 x 8192 x 2048, 384 tiles, takes the
-    //  22 us of 512 tiles; whole rounds of CUs then)
+    // (the CUs that hold a second tile set the time: 192 x 8192 x 2048, 384 tiles, takes the 22 us of 512
+    //  tiles; whole rounds of CUs at such a K, halfway there at a short one: 16 x 19 456 x 896, 304 tiles,
+    //  10.6 us, 1024 x 1152 x 896, 288 tiles, 9.5 us)
     const int cus = device_info().cus;
-    const long counted = nk >= 20 && t64 > cus ? (t64 + cus - 1) / cus * cus : t64;
+    const long rounds = (t64 + cus - 1) / cus * cus;
+    const long counted = t64 <= cus ? t64 : nk >= 20 ? rounds : (t64 + rounds) / 2;
     const double bulk = 3.3 + counted * nk * (nk > 32 ? 0.00155 : 0.0012);
     return serial > bulk ? serial : bulk;
 }
