@@ -926,8 +926,12 @@ int pick_vl(WeightKind kind, int M, long rows, int K) {
     // 15.0, K = 4608 25.6 / 22.0 / 14.4, K = 2560 11.3 / 9.8 / 9.6; Q4 K = 4608 17.0 / 13.5 / 11.6, K = 2560
     // 7.6 / 7.8 / 8.2; fp16 K = 4864 - / 28.8 / 27.2.  (The kernel with x in LDS, for every other long K,
     // keeps the wide tile: int8 16 384 x 4096 in 18.8 / 19.3 / 25.3 us.)
+    // K = 1536, int8 and fp16: 32 768 rows 13.6 / 11.1 / 10.5 us, 49 152 rows 16.7 / 14.6 / 14.4 us (int8), fp16
+    // 18.3 / 17.4 and 25.1 / 24.3 us at two / one; Q4 there, and every kind at K = 1024 and 576, is fastest
+    // with four.
     if (K == 4608 || K == 4864) max_vl = 1;
     else if (K == 2560 && kind != WK_Q4) max_vl = 2;
+    else if (K == 1536 && kind != WK_Q4) max_vl = 1;
     const long waves_wanted = 4L * device_info().cus;
     int narrowest = 1;
     for (int vl = max_vl; vl >= 1; vl >>= 1) {
