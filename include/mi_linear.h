@@ -168,7 +168,8 @@ int   mi_graph_destroy(void* graph);
 /* Selects how M > 1 is computed: 0 (default) = MFMA GEMM with fused dequant for M >= 16, and
  * for 2 <= M < 16 where it is estimated to beat M rows of GEMV (each row streams W again; e.g. an
  * lm_head from M = 2, an MLP projection from M = 3 to 6, a projection of a million weights from
- * about 12); K not a multiple of 64 or operands not 16-byte aligned always take the batched GEMV; 1 = always the batched GEMV, whose rows
+ * about 12); K not a multiple of 64 or operands not 16-byte aligned always take the batched GEMV;
+ * 1 = always the batched GEMV, whose rows
  * are bit-identical to M = 1 calls (the reference's prefill loop, LF/src/model.cpp:243-250);
  * 2, 3 and 11..15 = as 0 with the kernel choice pinned (tests and tuning: results stay within
  * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel (int8 and fp16
