@@ -226,7 +226,28 @@ def test_streaming_gemm_is_not_the_choice_for_many_megabytes_of_weights(queue):
         xb = mil.Buffer(16 * K * 2)
         assert mil.nnopt_register_int8_weight(wb, sb, N, K)
         try:
-            assert mil.linear_plan(queue, 16, N, K, xb, wb)[0] == kernel, (N, K, mil.linear_plan(queue, 16, N, K, xb, wb))
+            plan = mil.linear_plan(queue, 16, N, K, xb, wb)
+            assert plan[0] == kernel, (N, K, plan)
+            if kernel == 1:
+                assert plan[1] == 32, plan                  # no tile taller than the 16 rows of x need
+        finally:
+            mil.nnopt_unregister_weight(wb)
+
+
+def test_plans_of_the_configured_prefill_shapes(queue):
+    """Which kernel the library's own choice is at the benchmark's int8 shapes (plans only): the wide
+    kernel in 64-row tiles at 512 x 4864 x 896, in 160-row tiles at 2048, in slices of K at N = 896, the
+    streaming kernel at 16 rows, rows of GEMV for two rows of an MLP projection."""
+    expect = {(512, 4864, 896): (1, 64, 1), (2048, 4864, 896): (1, 160, 1), (2048, 896, 4864): (1, 64, 2),
+              (16, 4864, 896): (4, 16, 4), (2, 4864, 896): (0, 0, 1)}
+    for (N, K) in ((4864, 896), (896, 4864)):
+        wb, sb = mil.Buffer(N * K), mil.Buffer(N * 2)
+        xb = mil.Buffer(2048 * K * 2)
+        assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+        try:
+            for (M, n, k), plan in expect.items():
+                if (n, k) == (N, K):
+                    assert mil.linear_plan(queue, M, N, K, xb, wb) == plan, (M, N, K, mil.linear_plan(queue, M, N, K, xb, wb))
         finally:
             mil.nnopt_unregister_weight(wb)
 
