@@ -137,6 +137,30 @@ def test_dequant_and_unpack_views_bit_exact(queue):
 
 
 @pytest.mark.parametrize("kind", ["i8", "q4", "f16"])
+def test_longest_rows(queue, kind, capfd):
+    """K = 32 768, the longest row the library takes (x fills 64 KB of LDS), bit for bit; one step more is
+    refused with an error line and nothing is written."""
+    N, K = 70, 32768
+    W, x = synth_w(900, N, K), synth_x(901, K)
+    if kind == "i8":
+        q, s = mil.quantize_int8(W)
+        got, want = _run_linear(queue, 1, N, K, x, q, s, "i8")[0], O.gemv_i8(x, q, s.view(np.uint16))
+    elif kind == "q4":
+        p, sc = mil.quantize_q4(W)
+        got, want = _run_linear(queue, 1, N, K, x, p, sc, "q4")[0], O.gemv_q4(x, p, sc.view(np.uint16))
+    else:
+        got, want = _run_linear(queue, 1, N, K, x, W)[0], O.gemv_f16(x, W)
+    assert np.array_equal(got, want), f"{np.count_nonzero(got != want)} of {N} differ"
+    K2 = K + 32
+    xb, wb, ob = mil.Buffer(K2 * 2), mil.Buffer(4 * K2 * 2), mil.Buffer.from_host(np.full(4, 0x7BCD, np.uint16))
+    capfd.readouterr()
+    assert not mil.pytorch_linear(queue, 1, 4, K2, xb, wb, ob)
+    queue.finish()
+    assert "ERROR:" in capfd.readouterr().err
+    assert np.all(ob.read(np.uint16, (4,)) == 0x7BCD)
+
+
+@pytest.mark.parametrize("kind", ["i8", "q4", "f16"])
 def test_small_batches_are_rows_of_gemv(queue, kind):
     M, N, K = 5, 1000, 896
     W, X = synth_w(13, N, K), synth_x(14, M, K)
