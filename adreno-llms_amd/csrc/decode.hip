@@ -268,9 +268,20 @@ __global__ __launch_bounds__(256) void rope_attention_kernel(const uint16_t* __r
 // output element, keys in index order from the tile.  Longer contexts take further tiles the
 // same way, one round trip per 128 rows.  The arithmetic and its order are those of
 // rope_attention_kernel.
-// Dynamic LDS: 6 D bytes, 6 bytes per position, rounded up to 16, then two tiles of
-// kTileRows x (2 D + 16) bytes.
+// The two serial chains the order of operations leaves (the sum of the exponentials by one lane, an
+// output element's sum over the keys by one lane each) run in batches of kBatch positions: all LDS
+// reads of a batch are asked for together and the dependent additions follow as they arrive, so a
+// batch costs one LDS round trip and not one per position.  The last batch is filled up with
+// zeros (exponentials past the last key, probabilities from the current position on, value rows
+// from the current position on), which leaves a sum as it is: x + 0 = x and fma(0, 0, x) = x for
+// every x but -0, and a sum that starts at +0 never becomes -0.  The current position's
+// probability is kept aside (pc) and meets the current value row after the tiles, as before.
+// Dynamic LDS: 6 D bytes, 6 bytes per position (positions rounded up to kBatch), 16 bytes, then two
+// tiles of kTileRows x (2 D + 16) bytes.
 constexpr int kTileRows = 128;
+constexpr int kBatch = 32;
+static_assert(kTileRows % kBatch == 0, "whole batches in a tile");
+__host__ __device__ inline int padded_positions(int max_pos) { return (max_pos + kBatch - 1) / kBatch * kBatch; }
 constexpr int kMaxPositions = 8192;                      // longest context a decoder is created for
 
 template <int D>
@@ -292,82 +303,111 @@ __global__ __launch_bounds__(256) void rope_attention_tiled(uint16_t* __restrict
     extern __shared__ __attribute__((aligned(16))) uint16_t qv[];
     uint16_t* kcur = qv + D;
     uint16_t* vcur = kcur + D;
-    float* ex = reinterpret_cast<float*>(vcur + D);                        // [max_pos] exponentials
-    uint16_t* sc = reinterpret_cast<uint16_t*>(ex + max_pos);              // [max_pos] scores
-    uint16_t* ktile = qv + ((3 * D + 3 * max_pos + 7) & ~7);               // 16-byte aligned
+    const int mp = padded_positions(max_pos);
+    float* ex = reinterpret_cast<float*>(vcur + D);                        // [mp] exponentials, 16-byte aligned
+    uint16_t* sc = reinterpret_cast<uint16_t*>(ex + mp);                   // [mp] scores, 16-byte aligned
+    uint16_t* pc = sc + mp;                                                // the current position's probability
+    uint16_t* ktile = pc + 8;                                              // 16-byte aligned
     uint16_t* vtile = ktile + kTileRows * kRowH;
     const int nrep = n_heads / n_kv_heads;
     const int qh = blockIdx.x, kvd = n_kv_heads * D, kvh = qh / nrep, hd2 = D / 2;
     const bool writer = qh % nrep == 0;
     const int tid = threadIdx.x;
 
-    // piece p of this thread in a tile: row (tid + 256 p) / kPieces, 16-byte piece (tid + 256 p) % kPieces
-    auto request = [&](const uint16_t* cache, int row0, u32x4 (&r)[kPasses]) {
-        #pragma unroll
-        for (int p = 0; p < kPasses; ++p) {
-            const int idx = tid + 256 * p, row = idx / kPieces, piece = idx % kPieces;
-            const int tk = row0 + row < max_pos ? row0 + row : max_pos - 1;
-            r[p] = *reinterpret_cast<const u32x4*>(cache + static_cast<size_t>(tk) * kvd + kvh * D + 8 * piece);
-        }
-    };
-    auto keep = [&](uint16_t* tile, const u32x4 (&r)[kPasses]) {
-        #pragma unroll
-        for (int p = 0; p < kPasses; ++p) {
-            const int idx = tid + 256 * p, row = idx / kPieces, piece = idx % kPieces;
-            *reinterpret_cast<u32x4*>(tile + row * kRowH + 8 * piece) = r[p];
-        }
+    // piece p of this thread in a tile: row (tid + 256 p) / kPieces, 16-byte piece (tid + 256 p) % kPieces;
+    // pass p of all threads is rows p kPassRows .. (p + 1) kPassRows - 1.  Passes are asked for in
+    // row order, keys and values alternating, and loads return in the order of the requests: a
+    // short context waits for its first passes only and leaves the rest to arrive unused.
+    constexpr int kPassRows = 256 / kPieces;
+    auto request = [&](const uint16_t* cache, int row0, int p) {
+        const int idx = tid + 256 * p, row = idx / kPieces, piece = idx % kPieces;
+        const int tk = row0 + row < max_pos ? row0 + row : max_pos - 1;
+        return *reinterpret_cast<const u32x4*>(cache + static_cast<size_t>(tk) * kvd + kvh * D + 8 * piece);
     };
     u32x4 kreg[kPasses], vreg[kPasses];
-    request(kc, 0, kreg);
-    request(vc, 0, vreg);
-
+    auto request_tiles = [&](int row0, int first_pass) {
+        #pragma unroll
+        for (int p = first_pass; p < kPasses; ++p) {
+            kreg[p] = request(kc, row0, p);
+            vreg[p] = request(vc, row0, p);
+            asm volatile("" ::: "memory");                 // in this order: the compiler would sort them by cache
+        }
+    };
+    // the passes that hold rows below `rows` (of kBatch; the value sums run in whole batches) go to
+    // LDS; value rows from row `valid` of the tile on are stored as zeros
+    auto keep = [&](uint16_t* tile, const u32x4 (&r)[kPasses], int rows, int valid) {
+        #pragma unroll
+        for (int p = 0; p < kPasses; ++p) {
+            if (p * kPassRows < rows) {
+                const int idx = tid + 256 * p, row = idx / kPieces, piece = idx % kPieces;
+                const u32x4 zero = {0u, 0u, 0u, 0u};
+                *reinterpret_cast<u32x4*>(tile + row * kRowH + 8 * piece) = row < valid ? r[p] : zero;
+            }
+        }
+    };
+    // rows of the tile at row0 that anybody reads: the keys below the current position, in whole batches
+    auto tile_rows = [&](int row0, int pos) {
+        const int n = pos - row0 < kTileRows ? pos - row0 : kTileRows;
+        return (n + kBatch - 1) / kBatch * kBatch;
+    };
+    // The tiles' first passes are asked for first: their addresses need nothing but the arguments that
+    // arrive in registers.  What the current position needs (projections, biases, the rotary row: a few
+    // bytes per thread, behind pointers that have to be fetched) is asked for next, ahead of the other
+    // passes, and arrives ahead of them, so that q, k and v are prepared while the tiles come in.  Wavefront 0 prepares q, 1 k, 2 and 3 v; every thread loads from a valid
+    // address whether it has an element or not, so the number of loads in flight is the same for all.
     int pos = st->pos;
+    kreg[0] = request(kc, 0, 0);
+    vreg[0] = request(vc, 0, 0);
+    asm volatile("" ::: "memory");
+    const int role = tid >> 6, lane = tid & 63;
+    const int i = role < 2 ? (lane < hd2 ? lane : hd2 - 1) : (tid - 128 < D ? tid - 128 : D - 1);
+    const int i2 = role < 2 ? i + hd2 : i;
+    const uint16_t* buf = role == 0 ? q_raw + qh * D : role == 1 ? k_raw + kvh * D : v_raw + kvh * D;
+    const uint16_t* bias = role == 0 ? bq + qh * D : role == 1 ? bk + kvh * D : bv + kvh * D;
+    const uint16_t raw1 = buf[i], raw2 = buf[i2], bias1 = bias[i], bias2 = bias[i2];
+    const uint16_t cos_i = rope_now[role < 2 ? i : 0], sin_i = rope_now[D + (role < 2 ? i : 0)];   // embed_kernel's row
+    asm volatile("" ::: "memory");                             // these first
+    request_tiles(0, 1);
+    __builtin_amdgcn_sched_barrier(0);                         // and nothing that waits for one of them in between
+
     pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
     const int seq_k = pos + 1;
-    const uint16_t* cr = rope_now;                          // the rotary row of this position (embed_kernel)
-    const uint16_t* sr = rope_now + D;
-    if (tid < hd2) {
-        const int i = tid;
-        const float c = h_f(cr[i]), sn = h_f(sr[i]);
-        {
-            const uint16_t* buf = q_raw + qh * D;
-            const uint16_t* bias = bq + qh * D;
-            const float x1 = h_f(f_h(h_f(buf[i]) + h_f(bias[i])));
-            const float x2 = h_f(f_h(h_f(buf[i + hd2]) + h_f(bias[i + hd2])));
-            const uint16_t r1 = f_h(fmaf(x1, c, -(x2 * sn))), r2 = f_h(fmaf(x2, c, x1 * sn));
-            qv[i] = r1;
-            qv[i + hd2] = r2;
+    // (computed by every thread, stored by those that have an element: a load that is only used under a
+    //  condition would be moved there, behind the tiles)
+    const float c = h_f(cos_i), sn = h_f(sin_i);
+    const float x1 = h_f(f_h(h_f(raw1) + h_f(bias1)));
+    const float x2 = h_f(f_h(h_f(raw2) + h_f(bias2)));
+    const uint16_t r1 = f_h(fmaf(x1, c, -(x2 * sn))), r2 = f_h(fmaf(x2, c, x1 * sn));
+    const bool has_pair = role < 2 && lane < hd2, has_v = role >= 2 && tid - 128 < D;
+    const uint16_t rv = f_h(x1);                               // fp16(v + bias), rounded once
+    if (has_pair) {
+        uint16_t* dst = role == 0 ? qv : kcur;
+        dst[i] = r1;
+        dst[i + hd2] = r2;
+    } else if (has_v) {
+        vcur[tid - 128] = rv;
+    }
+    keep(ktile, kreg, tile_rows(0, pos), kTileRows);
+    keep(vtile, vreg, tile_rows(0, pos), pos);
+    // (the stores to memory after the tiles are in LDS: a store in flight counts like a load that has not
+    //  arrived, and would make the waits above wait for later passes than they need)
+    if (has_pair) {
+        if (role == 0) {
             q_out[qh * D + i] = r1;
             q_out[qh * D + i + hd2] = r2;
-        }
-    } else if (tid >= 64 && tid < 64 + hd2) {
-        const int i = tid - 64;
-        const float c = h_f(cr[i]), sn = h_f(sr[i]);
-        const uint16_t* buf = k_raw + kvh * D;
-        const uint16_t* bias = bk + kvh * D;
-        const float x1 = h_f(f_h(h_f(buf[i]) + h_f(bias[i])));
-        const float x2 = h_f(f_h(h_f(buf[i + hd2]) + h_f(bias[i + hd2])));
-        const uint16_t r1 = f_h(fmaf(x1, c, -(x2 * sn))), r2 = f_h(fmaf(x2, c, x1 * sn));
-        kcur[i] = r1;
-        kcur[i + hd2] = r2;
-        if (writer) {
+        } else if (writer) {
             uint16_t* dst = kc + static_cast<size_t>(pos) * kvd + kvh * D;
             dst[i] = r1;
             dst[i + hd2] = r2;
             k_out[kvh * D + i] = r1;
             k_out[kvh * D + i + hd2] = r2;
         }
-    } else if (tid >= 128 && tid < 128 + D) {
+    } else if (has_v && writer) {
         const int e = tid - 128;
-        const uint16_t r = f_h(h_f(v_raw[kvh * D + e]) + h_f(bv[kvh * D + e]));
-        vcur[e] = r;
-        if (writer) {
-            vc[static_cast<size_t>(pos) * kvd + kvh * D + e] = r;
-            v_out[kvh * D + e] = r;
-        }
+        vc[static_cast<size_t>(pos) * kvd + kvh * D + e] = rv;
+        v_out[kvh * D + e] = rv;
     }
-    keep(ktile, kreg);
-    keep(vtile, vreg);
+    if (pos > kTileRows) request_tiles(kTileRows, 0);          // the second tiles, one tile ahead of their use
     __syncthreads();
 
     // scores: tile rows by threads 0 .. kTileRows - 1, the current position by thread kTileRows
@@ -390,9 +430,12 @@ __global__ __launch_bounds__(256) void rope_attention_tiled(uint16_t* __restrict
     if (tid == kTileRows) sc[pos] = score(kcur);
     for (int row0 = 0; row0 < pos; row0 += kTileRows) {
         if (row0 > 0) {
-            request(kc, row0, kreg);
             __syncthreads();                               // the previous tile's scores are done
-            keep(ktile, kreg);
+            keep(ktile, kreg, tile_rows(row0, pos), kTileRows);
+            if (row0 + kTileRows < pos) {
+                #pragma unroll
+                for (int p = 0; p < kPasses; ++p) kreg[p] = request(kc, row0 + kTileRows, p);
+            }
             __syncthreads();
         }
         if (tid < kTileRows && row0 + tid < pos) sc[row0 + tid] = score(ktile + tid * kRowH);
@@ -409,34 +452,67 @@ __global__ __launch_bounds__(256) void rope_attention_tiled(uint16_t* __restrict
             ex[c] = e;
             sc[c] = f_h(e);
         }
+        const int padded = (seq_k + kBatch - 1) / kBatch * kBatch;
+        if (tid < padded - seq_k) ex[seq_k + tid] = 0.0f;      // kBatch <= 64 lanes
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");  // lane 0 reads what the other lanes wrote
         __builtin_amdgcn_wave_barrier();
         float inv = 0.0f;
         if (tid == 0) {
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+            const f32x4* e4 = reinterpret_cast<const f32x4*>(ex);
             float sum = 0.0f;
-            for (int c = 0; c < seq_k; ++c) sum = sum + ex[c];
+            for (int c = 0; c < padded; c += kBatch) {
+                f32x4 t[kBatch / 4];
+                #pragma unroll
+                for (int j = 0; j < kBatch / 4; ++j) t[j] = e4[c / 4 + j];
+                #pragma unroll
+                for (int j = 0; j < kBatch / 4; ++j) {
+                    sum = sum + t[j][0];
+                    sum = sum + t[j][1];
+                    sum = sum + t[j][2];
+                    sum = sum + t[j][3];
+                }
+            }
             inv = rcp_rn(sum + 1e-20f);
         }
         inv = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(inv)));
-        for (int c = tid; c < seq_k; c += 64) sc[c] = f_h(h_f(sc[c]) * inv);
+        // probabilities of the older keys; zeros from the current position to the end of its batch
+        for (int c = tid; c < padded; c += 64) {
+            const uint16_t pr = f_h(h_f(sc[c]) * inv);
+            if (c == pos) pc[0] = pr;
+            sc[c] = c < pos ? pr : static_cast<uint16_t>(0);
+        }
     }
     __syncthreads();
     // output element e by thread e: older keys in index order from the tiles, then the current one
     float acc = 0.0f;
     for (int row0 = 0; row0 < pos; row0 += kTileRows) {
         if (row0 > 0) {
-            request(vc, row0, vreg);
             __syncthreads();                               // the previous tile has been used up
-            keep(vtile, vreg);
+            keep(vtile, vreg, tile_rows(row0, pos), pos - row0);
+            if (row0 + kTileRows < pos) {
+                #pragma unroll
+                for (int p = 0; p < kPasses; ++p) vreg[p] = request(vc, row0 + kTileRows, p);
+            }
             __syncthreads();
         }
         if (tid < D) {
+            typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
             const int n = pos - row0 < kTileRows ? pos - row0 : kTileRows;
-            for (int r = 0; r < n; ++r) acc = fmaf(h_f(sc[row0 + r]), h_f(vtile[r * kRowH + tid]), acc);
+            for (int r0 = 0; r0 < n; r0 += kBatch) {
+                u16x8 p[kBatch / 8];
+                uint16_t v[kBatch];
+                #pragma unroll
+                for (int j = 0; j < kBatch / 8; ++j) p[j] = *reinterpret_cast<const u16x8*>(sc + row0 + r0 + 8 * j);
+                #pragma unroll
+                for (int u = 0; u < kBatch; ++u) v[u] = vtile[(r0 + u) * kRowH + tid];
+                #pragma unroll
+                for (int u = 0; u < kBatch; ++u) acc = fmaf(h_f(p[u / 8][u % 8]), h_f(v[u]), acc);
+            }
         }
     }
     if (tid < D) {
-        acc = fmaf(h_f(sc[pos]), h_f(vcur[tid]), acc);
+        acc = fmaf(h_f(pc[0]), h_f(vcur[tid]), acc);
         out[qh * D + tid] = f_h(acc);
     }
 }
@@ -891,7 +967,7 @@ __global__ void set_pos_kernel(State* st, int pos) { st->pos = pos; }
 
 // Dynamic LDS of rope_attention_tiled<D>.
 inline size_t tiled_attention_lds(int D, int max_pos) {
-    const size_t head = (static_cast<size_t>(3 * D + 3 * max_pos + 7) & ~static_cast<size_t>(7)) * 2;
+    const size_t head = static_cast<size_t>(3 * D + 3 * padded_positions(max_pos) + 8) * 2;
     return head + 2 * static_cast<size_t>(kTileRows) * (D + 8) * 2;
 }
 
