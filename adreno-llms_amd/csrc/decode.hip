@@ -259,14 +259,15 @@ __global__ __launch_bounds__(256) void rope_attention_kernel(const uint16_t* __r
 // The same launch for head widths known at compile time (64 and 128), laid out for latency: a
 // decode step at a short context is a chain of memory round trips, so everything that does not
 // depend on an earlier result is requested at once.  256 threads; the first kTileRows rows of the
-// group's key and value cache are requested in 16-byte pieces before anything else (rows past
+// group's key and value cache are requested in 16-byte pieces, in passes of 256 pieces (rows past
 // the current position too: the caches hold max_pos rows, and what is not older than the current
-// position is never used), then the projections, biases and the rotary row (which the step's first
+// position is never used; the passes above it are neither waited for nor kept), and between the
+// first pass and the others the projections, biases and the rotary row (which the step's first
 // launch has set aside, so that its address does not wait for the position); keys and values wait
 // in LDS tiles (rows padded by 16 bytes against bank conflicts) while q, k and v of the current
 // position are prepared.  Scores: one thread per key from the tile; values: one thread per
 // output element, keys in index order from the tile.  Longer contexts take further tiles the
-// same way, one round trip per 128 rows.  The arithmetic and its order are those of
+// same way, each requested while the one before it is used.  The arithmetic and its order are those of
 // rope_attention_kernel.
 // The two serial chains the order of operations leaves (the sum of the exponentials by one lane, an
 // output element's sum over the keys by one lane each) run in batches of kBatch positions: all LDS
