@@ -604,3 +604,44 @@ def test_modes_belong_to_the_stream_that_set_them(queue):
         L.mi_set_gemm_mode(0)
         L.mi_stream_set_modes(other.handle, -1, -1)
         mil.nnopt_unregister_weight(wb)
+
+
+# (N, K) of the projections of the three model families the reference ships (stacked q | k | v and
+# gate | up as a prompt runs them), and rows of x from a few tokens to a long prompt
+_MODEL_PROJECTIONS = [(1152, 896), (896, 896), (9728, 896), (896, 4864),              # Qwen2.5-0.5B
+                      (960, 576), (576, 576), (3072, 576), (576, 1536),               # SmolLM2-135M
+                      (1536, 1024), (1024, 1024), (9216, 1024), (1024, 4608),         # LFM2-350M
+                      (2560, 1024), (8192, 2048)]
+_PROMPT_ROWS = [24, 48, 96, 192, 384, 640, 1024, 1536, 2048, 4096]
+
+
+@pytest.mark.parametrize("kind", ["i8", "f16", "q4"])
+def test_planned_kernels_at_model_shapes(queue, kind):
+    """The library's own choice of kernel, tile height and K slices (mode 0) at the shapes its fitted
+    time estimates were tuned on, two prompt lengths per projection: every element against the
+    rows-of-GEMV mode of the same entry point, which the GEMV tests hold to the oracle bit for bit
+    (int8, fp16) or within the stated tolerance (Q4)."""
+    seen = set()
+    for i, (N, K) in enumerate(_MODEL_PROJECTIONS):
+        W = synth_w(5000 + i, N, K)
+        if kind == "i8":
+            w_host, s_host = mil.quantize_int8(W)
+        elif kind == "q4":
+            w_host, s_host = mil.quantize_q4(W)
+        else:
+            w_host, s_host = W, None
+        for j in range(2):
+            M = _PROMPT_ROWS[(3 * i + 5 * j + len(kind)) % len(_PROMPT_ROWS)]
+            if M * N > 12_000_000:                          # (bounds the rows-of-GEMV launch)
+                M = 256
+            X = synth_x(5100 + 2 * i + j, M, K)
+            plan = []
+            got = _gemm(queue, M, N, K, X, w_host, s_host, kind, plan=plan)
+            print(f"{kind} M={M} N={N} K={K} plan {plan[0]}", flush=True)
+            seen.add(plan[0][0])
+            rows = _gemm(queue, M, N, K, X, w_host, s_host, kind, tile=1)
+            assert_tolerance(got.view(np.float16), rows.view(np.float16))
+            if kind != "q4":
+                assert _ulp_apart(got, rows).max() <= 1, (M, N, K, plan[0])
+                assert np.mean(got == rows) > 0.99, (M, N, K, plan[0])
+    assert 1 in seen and len(seen) >= 2, seen               # the wide tiles and at least one other kernel ran
