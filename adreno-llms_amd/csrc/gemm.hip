@@ -811,11 +811,12 @@ inline double estimate_us(int kind, int terms, int tm, int splits, int M, int N,
     const double round = q4_tall ? 1.25 : 1.56;
     double t = full * round * block_us + (rem ? (1.0 + crowd * rem / slots) * block_us : 0.0);
     // every row of tiles streams W again: not faster than that many bytes at about 6.8 TB/s, or,
-    // for a W that stays in the memory-side cache (32 MB taken as the limit), 2.2 times that for
+    // for a W that stays in the memory-side cache (40 MB taken as the limit: fp16 8192 x 2048, 33.5 MB, still
+    // runs eight rows of tiles in 25.9 us, and the choices at 50 MB and more are right as they are), 2.2 times that for
     // the reads after the first
     const double w_once = static_cast<double>(N) * K * (kind == WK_F16 ? 2.0 : kind == WK_I8 ? 1.0 : 0.5625);
     const int tiles_m = (M + 32 * tm - 1) / (32 * tm);
-    const double w_bytes = w_once <= 32.0e6 ? w_once * (1.0 + (tiles_m - 1) / 2.2) : w_once * tiles_m;
+    const double w_bytes = w_once <= 40.0e6 ? w_once * (1.0 + (tiles_m - 1) / 2.2) : w_once * tiles_m;
     if (t < 2.5 + w_bytes / 6.8e6) t = 2.5 + w_bytes / 6.8e6;
     if (splits > 1) t += 2.5 + 2.0 * splits * M * static_cast<double>(N) * 4 / 4.0e6;   // ~4 TB/s there and back
     return t;
