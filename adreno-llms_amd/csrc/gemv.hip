@@ -930,7 +930,7 @@ int pick_vl(WeightKind kind, int M, long rows, int K) {
     // 18.3 / 17.4 and 25.1 / 24.3 us at two / one; Q4 there, and every kind at K = 1024 and 576, is fastest
     // with four.
     if (K == 4608 || K == 4864) max_vl = 1;
-    else if (K == 2560 && kind != WK_Q4) max_vl = 2;
+    else if ((K == 2560 || K == 2048) && kind != WK_Q4) max_vl = 2;
     else if (K == 1536 && kind != WK_Q4) max_vl = 1;
     const long waves_wanted = 4L * device_info().cus;
     int narrowest = 1;
@@ -1036,6 +1036,8 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
         MI_FIXED(896, true)
         MI_FIXED(1024, true)
         MI_FIXED(1536, true)
+        MI_FIXED(2048, false)         // the width of the 1-2 B models of the same families: the kernel with x in LDS
+                                      // took 27.3 us for int8 65 536 x 2048 where this one takes 24.0 (Q4: 38.1 -> 16.0)
         MI_FIXED(2560, false)         // LFM2's K values beside 1024: the reference ships kernels for exactly these
         MI_FIXED(4608, false)         // (LF/kernels/gemv_m1_int8.cl:155-255, gemv_m1_q4.cl:128-281)
         MI_FIXED(4864, false)
@@ -1106,6 +1108,8 @@ bool launch_q4_fast(hipStream_t s, const GemvCall* calls, int n, bool* taken) {
         MI_Q4F(896, false)
         MI_Q4F(1024, false)
         MI_Q4F(1536, false)
+        MI_Q4F(2048, false)
+        MI_Q4F(2560, false)
         default: *taken = false; return true;
     }
 #undef MI_Q4F

@@ -15,10 +15,10 @@ pytestmark = pytest.mark.gpu
 SHAPES_I8 = [(1536, 576), (576, 1536), (4864, 896), (896, 4864), (128, 896), (896, 896), (1152, 896),
              (4608, 1024), (1024, 4608), (1024, 2560), (37, 896), (5, 256), (1001, 1024), (3, 4864),
              (64, 320), (13, 36), (7, 4), (2049, 2048), (9, 8200),
-             (4100, 4864), (4099, 4608), (8200, 2560), (20001, 1536)]      # long rows, enough of them for any lane tile
+             (4100, 4864), (4099, 4608), (8200, 2560), (20001, 1536), (8200, 2048)]   # long rows, enough of them for any lane tile
 SHAPES_Q4 = [(4864, 896), (896, 4864), (128, 896), (4608, 1024), (1024, 4608), (1024, 2560), (37, 896),
              (5, 256), (3, 32), (64, 320), (11, 96), (1001, 1024), (9, 8192),
-             (4100, 4864), (4099, 4608), (8200, 2560)]
+             (4100, 4864), (4099, 4608), (8200, 2560), (8200, 2048), (37, 2048)]
 
 
 @pytest.fixture(scope="module")

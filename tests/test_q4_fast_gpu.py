@@ -39,7 +39,8 @@ def _run(queue, N, K, x, p, sc, add_to=None):
     return full[pad:-pad]
 
 
-@pytest.mark.parametrize("N,K", [(4864, 896), (151936, 896), (4608, 1024), (8192, 576), (4100, 1536), (4099, 896)])
+@pytest.mark.parametrize("N,K", [(4864, 896), (151936, 896), (4608, 1024), (8192, 576), (4100, 1536), (4099, 896),
+                                 (8192, 2048), (4101, 2048), (4100, 2560)])
 def test_fast_q4_within_tolerance(queue, N, K):
     print(f"fast q4 N={N} K={K}", flush=True)
     W, x = synth_w(1000 + N, N, K), synth_x(1100 + K, K)
@@ -47,13 +48,15 @@ def test_fast_q4_within_tolerance(queue, N, K):
     got = _run(queue, N, K, x, p, sc)
     want = O.gemv_q4(x, p, sc.view(np.uint16))
     assert_tolerance(got.view(np.float16), want.view(np.float16))
-    assert np.mean(got == want) > 0.97          # nearly all outputs are the same half
+    # nearly all outputs are the same half (a longer row has more additions whose order differs)
+    assert np.mean(got == want) > (0.97 if K <= 1536 else 0.94)
 
 
-def test_fast_q4_exact_on_integer_data_and_all_bytes(queue):
+@pytest.mark.parametrize("K", [896, 2048, 2560])
+def test_fast_q4_exact_on_integer_data_and_all_bytes(queue, K):
     # integer activations and power-of-two scales: every order of the fp32 sum is exact
     rng = np.random.default_rng(5)
-    N, K = 4096, 896
+    N = 4096
     p = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
     p[0, :256] = np.arange(256, dtype=np.uint8)
     sc = (2.0 ** rng.integers(-8, -3, (N, K // 32))).astype(np.float16)
