@@ -702,9 +702,47 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const uint16_t* x, int K) 
     for (int i = 2 * base + static_cast<int>(threadIdx.x); i < K / 2; i += kBlock) xs[i] = reinterpret_cast<const uint32_t*>(x)[i];
 }
 
+// x for the Q4 throughput arithmetic (see gemv_q4_fast) into LDS by the whole block: a thread takes a
+// scale block of 32 activations at a time, pairs them as v_dot2_f32_f16 wants them against a lane's 16
+// weight bytes, and adds them up.  Layout, for `nit` K-iterations of 16 blocks: 16-byte piece q of block
+// 16 j + g at uint4 index (4 j + q) 16 + g (the 16 lanes of a row read consecutive pieces), then -8 sum(x)
+// of block b at float index 256 nit + b.  Blocks past K hold zeros.
+__device__ __forceinline__ void stage_x_paired(uint32_t* xs, const uint16_t* x, int K, int nit) {
+    u32x4* xq = reinterpret_cast<u32x4*>(xs);
+    float* m8 = reinterpret_cast<float*>(xs) + 256 * nit;
+    const int blocks = K / 32;
+    for (int b = threadIdx.x; b < 16 * nit; b += kBlock) {
+        uint32_t raw[16];
+        if (b < blocks) {
+            load_dwords<16, false>(raw, x + 32 * b);
+        } else {
+            #pragma unroll
+            for (int i = 0; i < 16; ++i) raw[i] = 0u;
+        }
+        float sx = 0.0f;
+        #pragma unroll
+        for (int i = 0; i < 16; ++i) sx += lo_f(raw[i]) + hi_f(raw[i]);
+        const int j = b / 16, g = b % 16;
+        #pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            u32x4 t;
+            t.x = __builtin_amdgcn_perm(raw[4 * d + 2], raw[4 * d + 0], 0x05040100u);
+            t.y = __builtin_amdgcn_perm(raw[4 * d + 2], raw[4 * d + 0], 0x07060302u);
+            t.z = __builtin_amdgcn_perm(raw[4 * d + 3], raw[4 * d + 1], 0x05040100u);
+            t.w = __builtin_amdgcn_perm(raw[4 * d + 3], raw[4 * d + 1], 0x07060302u);
+            xq[(4 * j + d) * 16 + g] = t;
+        }
+        m8[b] = -8.0f * sx;
+    }
+}
+constexpr size_t paired_x_lds(int K) { return static_cast<size_t>((K + 511) / 512) * 16 * 68; }
+
 // ---- K known at run time: x is staged once per block in LDS ------------------------
-template <int KIND, int VL, int EPI>
+// FAST (Q4, four rows per wavefront): the arithmetic of gemv_q4_fast, inside the stated tolerance, for
+// every K that kernel has no instance for (the exact order is bound by the vector ALU at about 2 TB/s).
+template <int KIND, int VL, int EPI, bool FAST = false>
 __global__ __launch_bounds__(kBlock) void gemv_any_k(MI_HOT_PARAMS, const SegList L, int K) {
+    static_assert(!FAST || (KIND == WK_Q4 && VL == 4), "the throughput arithmetic is Q4's, a scale block per lane");
     using T = WT<KIND>;
     constexpr int LPR = kWave / VL, RPW = VL;
     constexpr int EIT = kWave * T::EPV;
@@ -712,11 +750,13 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(MI_HOT_PARAMS, const SegLis
     constexpr int WD = VL * T::BPV / 4;
     constexpr int ITB = kWave * T::BPV;
     constexpr int kChunk = 8;                           // K-iterations per register buffer (at most 32 dwords per lane)
-    extern __shared__ uint32_t xs[];                    // K/2 dwords of packed fp16
+    extern __shared__ __attribute__((aligned(16))) uint32_t xs[];   // K/2 dwords of packed fp16 (FAST: see stage_x_paired)
 
     const int m = blockIdx.y;
     x += static_cast<size_t>(m) * K;
-    stage_x(xs, x, K);
+    const int nit = (K + EIT - 1) / EIT;
+    if constexpr (FAST) stage_x_paired(xs, x, K, nit);
+    else stage_x(xs, x, K);
     __syncthreads();
 
     const int lane = threadIdx.x % kWave;
@@ -725,7 +765,6 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(MI_HOT_PARAMS, const SegLis
     const int koff = g * VL * T::EPV;
     const Consts cst = make_consts();
     const size_t rowb = static_cast<size_t>(K) / T::EPV * T::BPV;
-    const int nit = (K + EIT - 1) / EIT;
 
     for (int rb = blockIdx.x * kWavesPerBlock + wave; rb < hnbatch; rb += gridDim.x * kWavesPerBlock) {
         const Seg sg = hW1 == nullptr ? Seg{hW0, hsc0, hy0, hN0, 0} : find_segment(L, rb);
@@ -762,14 +801,37 @@ __global__ __launch_bounds__(kBlock) void gemv_any_k(MI_HOT_PARAMS, const SegLis
             for (int u = 0; u < kChunk; ++u) {
                 const int j = j0 + u, k = j * EIT + koff;
                 if (j < nit && k < K) {
-                    uint32_t xr[XD];
-                    #pragma unroll
-                    for (int i = 0; i < XD; ++i) xr[i] = xs[k / 2 + i];
-                    float sf = 0.0f;
-                    if constexpr (KIND == WK_Q4) sf = h_f(sbuf[b][u]);
-                    #pragma unroll
-                    for (int v = 0; v < VL; ++v)
-                        acc[v] = vlane_step<KIND>(acc[v], &wbuf[b][u][v * T::BPV / 4], &xr[v * T::EPV / 2], sf, cst);
+                    if constexpr (FAST) {
+                        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                        uint32_t xp[4][4];
+                        #pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            const u32x4 t = reinterpret_cast<const u32x4*>(xs)[(4 * j + d) * 16 + g];
+                            xp[d][0] = t.x; xp[d][1] = t.y; xp[d][2] = t.z; xp[d][3] = t.w;
+                        }
+                        const float m8sx = reinterpret_cast<const float*>(xs)[256 * nit + 16 * j + g];
+                        float da = 0.0f, db = 0.0f;
+                        #pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            const uint32_t v = wbuf[b][u][d], v8 = v >> 8;
+                            da = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xp[d][0]), __builtin_bit_cast(h2, v & 0x000F000Fu), da, false);
+                            db = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xp[d][1]), __builtin_bit_cast(h2, v & 0x00F000F0u), db, false);
+                            da = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xp[d][2]), __builtin_bit_cast(h2, v8 & 0x000F000Fu), da, false);
+                            db = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xp[d][3]), __builtin_bit_cast(h2, v8 & 0x00F000F0u), db, false);
+                        }
+                        // sum over the block of x * (n - 8) = 2^24 da + 2^20 db - 8 sum(x), times the block's scale
+                        const float blk = fmaf(da, 16777216.0f, fmaf(db, 1048576.0f, m8sx));
+                        acc[0] = fmaf(blk, h_f(sbuf[b][u]), acc[0]);
+                    } else {
+                        uint32_t xr[XD];
+                        #pragma unroll
+                        for (int i = 0; i < XD; ++i) xr[i] = xs[k / 2 + i];
+                        float sf = 0.0f;
+                        if constexpr (KIND == WK_Q4) sf = h_f(sbuf[b][u]);
+                        #pragma unroll
+                        for (int v = 0; v < VL; ++v)
+                            acc[v] = vlane_step<KIND>(acc[v], &wbuf[b][u][v * T::BPV / 4], &xr[v * T::EPV / 2], sf, cst);
+                    }
                 }
             }
         };
@@ -1110,7 +1172,12 @@ bool launch_q4_fast(hipStream_t s, const GemvCall* calls, int n, bool* taken) {
         MI_Q4F(1536, false)
         MI_Q4F(2048, false)
         MI_Q4F(2560, false)
-        default: *taken = false; return true;
+        default: {
+            // every other K: the same arithmetic with x in LDS (where it fits the 64 KB a launch gets unasked)
+            const size_t lds = paired_x_lds(K);
+            if (lds > 65536) { *taken = false; return true; }
+            hipLaunchKernelGGL((gemv_any_k<WK_Q4, 4, EPI, true>), p.grid, dim3(kBlock), lds, s, MI_HOT_ARGS(x, p.L), p.L, K);
+        }
     }
 #undef MI_Q4F
     return MI_HIP_OK(hipGetLastError());

@@ -187,8 +187,8 @@ void mi_set_gemm_mode(int mode);
 /* Selects the M = 1 arithmetic.  0 = every GEMV evaluates the reference kernels' sum in the
  * reference's own order (results bit-identical to a literal evaluation of
  * LF/kernels/gemv_m1_q4.cl etc.).  1 (default) = as 0 for fp16 and int8, which are HBM-bound
- * either way; Q4 at the specialised K values runs a kernel that sums the same fp32 products
- * in another order, about twice as fast, within the tolerance the reference's own tests
+ * either way; Q4 matrices with enough rows to fill the chip four rows to a wavefront (about 4096)
+ * run a kernel that sums the same fp32 products in another order, about twice as fast, within the tolerance the reference's own tests
  * accept (cosine per layer), not bit-identical. */
 void mi_set_gemv_mode(int mode);
 

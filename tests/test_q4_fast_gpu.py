@@ -40,7 +40,10 @@ def _run(queue, N, K, x, p, sc, add_to=None):
 
 
 @pytest.mark.parametrize("N,K", [(4864, 896), (151936, 896), (4608, 1024), (8192, 576), (4100, 1536), (4099, 896),
-                                 (8192, 2048), (4101, 2048), (4100, 2560)])
+                                 (8192, 2048), (4101, 2048), (4100, 2560),
+                                 # K values without an instance of their own: the same arithmetic with x in LDS
+                                 (4100, 960), (4099, 1280), (4096, 3072), (4098, 4096), (4096, 8192), (4097, 11008),
+                                 (4096, 32), (4100, 30720)])
 def test_fast_q4_within_tolerance(queue, N, K):
     print(f"fast q4 N={N} K={K}", flush=True)
     W, x = synth_w(1000 + N, N, K), synth_x(1100 + K, K)
@@ -49,10 +52,10 @@ def test_fast_q4_within_tolerance(queue, N, K):
     want = O.gemv_q4(x, p, sc.view(np.uint16))
     assert_tolerance(got.view(np.float16), want.view(np.float16))
     # nearly all outputs are the same half (a longer row has more additions whose order differs)
-    assert np.mean(got == want) > (0.97 if K <= 1536 else 0.94)
+    assert np.mean(got == want) > (0.96 if K <= 1536 else 0.94 if K <= 2560 else 0.8)
 
 
-@pytest.mark.parametrize("K", [896, 2048, 2560])
+@pytest.mark.parametrize("K", [896, 2048, 2560, 960, 3072, 8192])
 def test_fast_q4_exact_on_integer_data_and_all_bytes(queue, K):
     # integer activations and power-of-two scales: every order of the fp32 sum is exact
     rng = np.random.default_rng(5)
@@ -68,12 +71,13 @@ def test_fast_q4_exact_on_integer_data_and_all_bytes(queue, K):
     assert np.array_equal(got, O.gemv_q4(x, p, sc.view(np.uint16)))
 
 
-def test_fast_q4_unit_vectors_and_subnormal_activations(queue):
-    N, K = 4096, 896
+@pytest.mark.parametrize("K", [896, 1280])
+def test_fast_q4_unit_vectors_and_subnormal_activations(queue, K):
+    N = 4096
     W = synth_w(1200, N, K)
     p, sc = mil.quantize_q4(W)
     nib = np.stack([p & 15, p >> 4], -1).reshape(N, K).astype(np.float32) - 8
-    for k in (0, 1, 4, 5, 31, 32, 511, 512, 895):
+    for k in (0, 1, 4, 5, 31, 32, 511, 512, 895, K - 1):
         x = np.zeros(K, np.float16)
         x[k] = 1.0
         want = (nib[:, k] * sc[:, k // 32].astype(np.float32)).astype(np.float16)
@@ -85,8 +89,9 @@ def test_fast_q4_unit_vectors_and_subnormal_activations(queue):
     assert_tolerance(got.view(np.float16), O.gemv_q4(x, p, sc.view(np.uint16)).view(np.float16))
 
 
-def test_fast_q4_residual_epilogue(queue):
-    N, K = 8192, 896
+@pytest.mark.parametrize("K", [896, 3072])
+def test_fast_q4_residual_epilogue(queue, K):
+    N = 8192
     W, x = synth_w(1300, N, K), synth_x(1301, K)
     res0 = synth_x(1302, N)
     p, sc = mil.quantize_q4(W)
