@@ -1086,6 +1086,7 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
                 MI_FIXED_AM(896, true)
                 MI_FIXED_AM(1024, true)
                 MI_FIXED_AM(1536, true)
+                MI_FIXED_AM(2048, false)
                 MI_FIXED_AM(4864, false)
                 default: MI_ERROR_FMT("gemv: no fused argmax for K=%d", K); return false;
             }
@@ -1130,6 +1131,7 @@ bool launch_swiglu_vl(hipStream_t s, const GemvCall* calls) {
         MI_SWIGLU(896)
         MI_SWIGLU(1024)
         MI_SWIGLU(1536)
+        MI_SWIGLU(2048)
         default: MI_ERROR_FMT("gemv: no SwiGLU epilogue for K=%d", calls[0].K); return false;
     }
 #undef MI_SWIGLU
@@ -1230,13 +1232,13 @@ int gemv_argmax_slots(const GemvCall& c) {
 }
 
 bool gemv_takes_swiglu(WeightKind, int K) {
-    return K == 576 || K == 896 || K == 1024 || K == 1536;
+    return K == 576 || K == 896 || K == 1024 || K == 1536 || K == 2048;
 }
 
 // The kernels that keep x in registers (every weight kind; Q4 through the exact kernel, not the
 // throughput one).
 bool gemv_takes_norm(WeightKind, int K) {
-    return K == 576 || K == 896 || K == 1024 || K == 1536 || K == 4864;
+    return K == 576 || K == 896 || K == 1024 || K == 1536 || K == 2048 || K == 4864;
 }
 
 bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
