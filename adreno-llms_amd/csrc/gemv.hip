@@ -1084,6 +1084,7 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
             switch (K) {
                 MI_FIXED_AM(576, true)
                 MI_FIXED_AM(896, true)
+                MI_FIXED_AM(960, true)
                 MI_FIXED_AM(1024, true)
                 MI_FIXED_AM(1536, true)
                 MI_FIXED_AM(2048, false)
@@ -1097,6 +1098,7 @@ bool launch_kind_vl(hipStream_t s, const GemvCall* calls, int n) {
     switch (K) {
         MI_FIXED(576, true)
         MI_FIXED(896, true)
+        MI_FIXED(960, true)           // SmolLM2-360M's width
         MI_FIXED(1024, true)
         MI_FIXED(1536, true)
         MI_FIXED(2048, false)         // the width of the 1-2 B models of the same families: the kernel with x in LDS
@@ -1129,6 +1131,7 @@ bool launch_swiglu_vl(hipStream_t s, const GemvCall* calls) {
     switch (calls[0].K) {
         MI_SWIGLU(576)
         MI_SWIGLU(896)
+        MI_SWIGLU(960)
         MI_SWIGLU(1024)
         MI_SWIGLU(1536)
         MI_SWIGLU(2048)
@@ -1160,6 +1163,7 @@ bool launch_q4_fast(hipStream_t s, const GemvCall* calls, int n, bool* taken) {
             switch (K) {
                 MI_Q4F(576, true)
                 MI_Q4F(896, true)
+                MI_Q4F(960, true)
                 MI_Q4F(1024, true)
                 MI_Q4F(1536, true)
                 default: *taken = false; return true;
@@ -1170,6 +1174,7 @@ bool launch_q4_fast(hipStream_t s, const GemvCall* calls, int n, bool* taken) {
     switch (K) {
         MI_Q4F(576, false)
         MI_Q4F(896, false)
+        MI_Q4F(960, false)
         MI_Q4F(1024, false)
         MI_Q4F(1536, false)
         MI_Q4F(2048, false)
@@ -1222,7 +1227,7 @@ bool gemv_takes_argmax(hipStream_t s, const GemvCall& c) {
     if (c.M != 1 || c.epi != EPI_STORE) return false;
     if (c.kind == WK_Q4)
         return !c.norm_w && gemv_mode(s) == 1 && pick_vl(c.kind, 1, c.N, c.K) == 4 &&
-               (c.K == 576 || c.K == 896 || c.K == 1024 || c.K == 1536);
+               (c.K == 576 || c.K == 896 || c.K == 960 || c.K == 1024 || c.K == 1536);
     return gemv_takes_norm(c.kind, c.K);
 }
 
@@ -1232,13 +1237,13 @@ int gemv_argmax_slots(const GemvCall& c) {
 }
 
 bool gemv_takes_swiglu(WeightKind, int K) {
-    return K == 576 || K == 896 || K == 1024 || K == 1536 || K == 2048;
+    return K == 576 || K == 896 || K == 960 || K == 1024 || K == 1536 || K == 2048;
 }
 
 // The kernels that keep x in registers (every weight kind; Q4 through the exact kernel, not the
 // throughput one).
 bool gemv_takes_norm(WeightKind, int K) {
-    return K == 576 || K == 896 || K == 1024 || K == 1536 || K == 2048 || K == 4864;
+    return K == 576 || K == 896 || K == 960 || K == 1024 || K == 1536 || K == 2048 || K == 4864;
 }
 
 bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {

@@ -119,8 +119,8 @@ int mi_unpack_q4_to_int8(void* stream, const void* W_q4, int N, int K, void* w8)
 int mi_argmax_f16(void* stream, const void* logits, int N, int num_partials, void* token_out);
 /* mi_linear with M = 1 followed by mi_argmax_f16 on its output: the lm_head of a greedy decode step
  * (QW/src/model.cpp:436-482).  logits [N] fp16 is written as by mi_linear, token_out as by
- * mi_argmax_f16 from those logits.  For int8 and fp16 weights with K in {576, 896, 1024, 1536, 2048, 4864},
- * and for Q4 weights where the throughput GEMV runs (gemv mode 1, K in {576, 896, 1024, 1536}, at
+ * mi_argmax_f16 from those logits.  For int8 and fp16 weights with K in {576, 896, 960, 1024, 1536, 2048, 4864},
+ * and for Q4 weights where the throughput GEMV runs (gemv mode 1, K in {576, 896, 960, 1024, 1536}, at
  * least 4096 rows), on a stream with a workspace, the GEMV's wavefronts also leave their best row
  * (same order of preference) and the second launch reduces those candidates, so the logits are not
  * read back; otherwise the two calls run one after the other. */

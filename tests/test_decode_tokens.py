@@ -198,6 +198,9 @@ def test_smollm_widths_fp16_and_q4_weights_on_device(kind):
                          max_pos=100, rms_eps=1e-6, rope_theta=10000.0), 90),
     ("head_dim_96", dict(hidden=576, inter=1536, n_heads=6, n_kv_heads=3, head_dim=96, n_layers=1, vocab=1024,
                          max_pos=70, rms_eps=1e-5, rope_theta=100000.0), 66),
+    # SmolLM2-360M's widths (K = 960 and 2560; 15 query heads over 5 key/value heads)
+    ("hidden_960", dict(hidden=960, inter=2560, n_heads=15, n_kv_heads=5, head_dim=64, n_layers=2, vocab=4096,
+                        max_pos=40, rms_eps=1e-5, rope_theta=100000.0), 34),
     # the width of the families' 1 to 2 B models: K = 2048 with the norm, the SwiGLU and the argmax fused
     ("hidden_2048", dict(hidden=2048, inter=1536, n_heads=16, n_kv_heads=4, head_dim=128, n_layers=2, vocab=4096,
                          max_pos=40, rms_eps=1e-5, rope_theta=130000.0), 34),

@@ -15,10 +15,10 @@ pytestmark = pytest.mark.gpu
 SHAPES_I8 = [(1536, 576), (576, 1536), (4864, 896), (896, 4864), (128, 896), (896, 896), (1152, 896),
              (4608, 1024), (1024, 4608), (1024, 2560), (37, 896), (5, 256), (1001, 1024), (3, 4864),
              (64, 320), (13, 36), (7, 4), (2049, 2048), (9, 8200),
-             (4100, 4864), (4099, 4608), (8200, 2560), (20001, 1536), (8200, 2048)]   # long rows, enough of them for any lane tile
+             (4100, 4864), (4099, 4608), (8200, 2560), (20001, 1536), (8200, 2048), (8200, 960), (2560, 960)]   # long rows, enough of them for any lane tile
 SHAPES_Q4 = [(4864, 896), (896, 4864), (128, 896), (4608, 1024), (1024, 4608), (1024, 2560), (37, 896),
              (5, 256), (3, 32), (64, 320), (11, 96), (1001, 1024), (9, 8192),
-             (4100, 4864), (4099, 4608), (8200, 2560), (8200, 2048), (37, 2048)]
+             (4100, 4864), (4099, 4608), (8200, 2560), (8200, 2048), (37, 2048), (8200, 960), (2560, 960)]
 
 
 @pytest.fixture(scope="module")
@@ -240,7 +240,7 @@ def test_silu_gate_epilogue(queue, kind, N, K):
 
 
 @pytest.mark.parametrize("kind", ["i8", "f16"])
-@pytest.mark.parametrize("N,K", [(1536, 576), (4864, 896), (50, 64), (130, 4104)])
+@pytest.mark.parametrize("N,K", [(1536, 576), (4864, 896), (50, 64), (130, 4104), (2560, 960), (8192, 2048)])
 def test_gate_up_silu_epilogue(queue, kind, N, K):
     Wg, Wu, x = synth_w(18, N, K), synth_w(19, N, K), synth_x(20, K)
     xb, ob = mil.Buffer.from_host(x), mil.Buffer(N * 2)

@@ -40,7 +40,7 @@ def _run(queue, N, K, x, p, sc, add_to=None):
 
 
 @pytest.mark.parametrize("N,K", [(4864, 896), (151936, 896), (4608, 1024), (8192, 576), (4100, 1536), (4099, 896),
-                                 (8192, 2048), (4101, 2048), (4100, 2560),
+                                 (8192, 2048), (4101, 2048), (4100, 2560), (49152, 960),
                                  # K values without an instance of their own: the same arithmetic with x in LDS
                                  (4100, 960), (4099, 1280), (4096, 3072), (4098, 4096), (4096, 8192), (4097, 11008),
                                  (4096, 32), (4100, 30720)])
