@@ -99,3 +99,28 @@ def test_fast_q4_residual_epilogue(queue, K):
     want = res0.view(np.uint16).copy()
     O.lib.orc_gemv_q4_add(O.u16(x), p, np.ascontiguousarray(sc.view(np.uint16)), want, N, K)
     assert_tolerance(got.view(np.float16), want.view(np.float16))
+
+
+@pytest.mark.parametrize("K", [896, 3072])
+def test_fast_q4_rows_of_a_small_batch_equal_single_calls(queue, K):
+    """Three rows of x in one call (each row a GEMV of its own, gemm mode 1) and the same rows one
+    call each: the same kernel either way, so the same bits; K with an instance of its own and K
+    through the kernel that keeps x in LDS."""
+    N, M = 4100, 3
+    W, X = synth_w(1400 + K, N, K), synth_x(1401 + K, M, K)
+    p, sc = mil.quantize_q4(W)
+    singles = np.stack([_run(queue, N, K, X[i], p, sc) for i in range(M)])
+    xb, pb, sb = mil.Buffer.from_host(X), mil.Buffer.from_host(p), mil.Buffer.from_host(sc)
+    ob = mil.Buffer(M * N * 2)
+    assert mil.nnopt_register_q4_weight(pb, sb, N, K)
+    mil.lib().mi_set_gemm_mode(1)
+    try:
+        assert mil.pytorch_linear(queue, M, N, K, xb, pb, ob)
+        queue.finish()
+    finally:
+        mil.lib().mi_set_gemm_mode(0)
+        mil.nnopt_unregister_weight(pb)
+    got = ob.read(np.uint16, (M, N))
+    assert np.array_equal(got, singles)
+    for i in range(M):
+        assert_tolerance(got[i].view(np.float16), O.gemv_q4(X[i], p, sc.view(np.uint16)).view(np.float16))
