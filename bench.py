@@ -301,6 +301,9 @@ def main():
             detail[key]["frac_of_read_probe"] = round(detail["read_probe_q4_lm_head_bytes"]["us"] / detail[key]["us"], 4)
         detail["c3_int8_gemv_151936x896"] = {"us": roofline["us_per_launch"], "GBps": roofline["achieved"],
                                              "frac_hbm": roofline["frac"], "bytes": lm_bytes}
+        # the same streaming structure on fp16 weights (no config asks for it at this size): what the launch
+        # reaches when the arithmetic per byte is a quarter of int8's in the reference's order
+        detail["fp16_gemv_151936x896"] = cold_gemv("f16", VOCAB, H, 3)
         # the fused epilogues at the boundary (int8, warm): residual add, gate/up + SwiGLU, w3 + silu_mul
         def fused_us(fn, n=32):
             fn()
