@@ -60,6 +60,7 @@ _SIGNATURES = {
     "mi_decoder_reset": (_i, [_vp, _vp, _i, _i]),
     "mi_decoder_set_token": (_i, [_vp, _vp, _i]),
     "mi_decoder_step": (_i, [_vp, _vp]),
+    "mi_decoder_set_attention_splits": (_i, [_vp, _i]),
     "mi_decoder_prefill": (_i, [_vp, _vp, C.POINTER(_i), _i, _i]),
     "mi_decoder_reserve_prompt": (_i, [_vp, _vp, _i]),
     "mi_decoder_read": (_i, [_vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
@@ -358,6 +359,10 @@ class Decoder:
 
     def step(self, queue):
         return bool(lib().mi_decoder_step(self.handle, _q(queue)))
+
+    def set_attention_splits(self, splits):
+        """0 / 1: the reference-order attention (default); 2..32: a head's keys split over that many blocks."""
+        return bool(lib().mi_decoder_set_attention_splits(self.handle, int(splits)))
 
     def prefill(self, queue, tokens, pos0=0):
         """A prompt at once (Model::forward with seq_len = len(tokens), QW/src/model.cpp:243-376)."""

@@ -518,6 +518,180 @@ __global__ __launch_bounds__(256) void rope_attention_tiled(uint16_t* __restrict
     }
 }
 
+// ---- attention with the keys of a head split over several blocks (an arithmetic mode, not the default) ----
+//
+// The launch above keeps the reference's order of operations, and at a long context that order is two
+// chains of dependent additions as long as the context, in one wavefront per head.  Here block (head, s) of
+// `splits` takes every splits-th run of the keys: scores as above (fp32 dot product, rounded to fp16 like
+// the reference's), its own maximum m, e = exp(score - m) in fp32, their sum l and o[d] = sum e v[d]; a
+// second launch merges the parts of a head: M = max m, out = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s.
+// The same real numbers as softmax(q k) v, summed in another order and without the fp16 roundings of the
+// probabilities: within the stated tolerance of the reference-order launch, not bit-identical.
+// part: [n_heads][splits][D + 2] floats: m, l, o[D].
+constexpr int kSplitThreads = 256;
+constexpr int kMaxSplits = 32;
+
+template <int D>
+__global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
+        uint16_t* __restrict__ kc, uint16_t* __restrict__ vc, const State* __restrict__ st, int n_heads, int n_kv_heads,
+        int max_pos, float scale, const uint16_t* __restrict__ q_raw, const uint16_t* __restrict__ k_raw,
+        const uint16_t* __restrict__ v_raw, const uint16_t* __restrict__ bq, const uint16_t* __restrict__ bk,
+        const uint16_t* __restrict__ bv, const uint16_t* __restrict__ rope_now, uint16_t* __restrict__ q_out,
+        uint16_t* __restrict__ k_out, uint16_t* __restrict__ v_out, float* __restrict__ part, int chunk_cap) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    float* sc = sm;                                            // [chunk_cap] scores, then exponentials
+    float* red = sc + chunk_cap;                               // [8] block reductions
+    float* osum = red + 8;                                     // [kSplitThreads / D][D] partial outputs
+    uint16_t* qv = reinterpret_cast<uint16_t*>(osum + kSplitThreads);   // [D] q, [D] k, [D] v of the current position
+    uint16_t* kcur = qv + D;
+    uint16_t* vcur = kcur + D;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int qh = blockIdx.x, sp = blockIdx.y, splits = gridDim.y;
+    const int nrep = n_heads / n_kv_heads, kvh = qh / nrep, kvd = n_kv_heads * D, hd2 = D / 2;
+    int pos = st->pos;
+    pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+    const int seq_k = pos + 1;
+    const int chunk = (seq_k + splits - 1) / splits;           // <= chunk_cap: the host sizes it for max_pos
+    const int k0 = sp * chunk, k1 = k0 + chunk < seq_k ? k0 + chunk : seq_k;
+    float* mine = part + (static_cast<size_t>(qh) * splits + sp) * (D + 2);
+    if (k0 >= k1) {                                            // no keys for this block at this position
+        if (tid == 0) { mine[0] = -3.402823466e+38f; mine[1] = 0.0f; }
+        if (tid < D) mine[2 + tid] = 0.0f;
+        return;
+    }
+    const bool has_current = k1 == seq_k;                      // the block whose run ends with the current position
+    // q of the head (every block), k and v of the current position (the block that needs them); the block of
+    // the group's first head also writes them to the caches and to the buffers a caller may inspect
+    if (tid < hd2) {
+        const float c = h_f(rope_now[tid]), sn = h_f(rope_now[D + tid]);
+        const float x1 = h_f(f_h(h_f(q_raw[qh * D + tid]) + h_f(bq[qh * D + tid])));
+        const float x2 = h_f(f_h(h_f(q_raw[qh * D + tid + hd2]) + h_f(bq[qh * D + tid + hd2])));
+        const uint16_t r1 = f_h(fmaf(x1, c, -(x2 * sn))), r2 = f_h(fmaf(x2, c, x1 * sn));
+        qv[tid] = r1;
+        qv[tid + hd2] = r2;
+        if (sp == 0) { q_out[qh * D + tid] = r1; q_out[qh * D + tid + hd2] = r2; }
+    } else if (has_current && tid >= 64 && tid < 64 + hd2) {
+        const int i = tid - 64;
+        const float c = h_f(rope_now[i]), sn = h_f(rope_now[D + i]);
+        const float x1 = h_f(f_h(h_f(k_raw[kvh * D + i]) + h_f(bk[kvh * D + i])));
+        const float x2 = h_f(f_h(h_f(k_raw[kvh * D + i + hd2]) + h_f(bk[kvh * D + i + hd2])));
+        const uint16_t r1 = f_h(fmaf(x1, c, -(x2 * sn))), r2 = f_h(fmaf(x2, c, x1 * sn));
+        kcur[i] = r1;
+        kcur[i + hd2] = r2;
+        if (qh % nrep == 0) {
+            uint16_t* dst = kc + static_cast<size_t>(pos) * kvd + kvh * D;
+            dst[i] = r1; dst[i + hd2] = r2;
+            k_out[kvh * D + i] = r1; k_out[kvh * D + i + hd2] = r2;
+        }
+    } else if (has_current && tid >= 128 && tid < 128 + D) {
+        const int e = tid - 128;
+        const uint16_t r = f_h(h_f(v_raw[kvh * D + e]) + h_f(bv[kvh * D + e]));
+        vcur[e] = r;
+        if (qh % nrep == 0) {
+            vc[static_cast<size_t>(pos) * kvd + kvh * D + e] = r;
+            v_out[kvh * D + e] = r;
+        }
+    }
+    __syncthreads();
+    // scores, a thread per key: the key's row straight from the cache (the current position's from LDS)
+    float m = -3.402823466e+38f;
+    for (int c = k0 + tid; c < k1; c += kSplitThreads) {
+        u32x4 kr[D / 8];
+        if (c == pos) {
+            #pragma unroll
+            for (int i = 0; i < D / 8; ++i) kr[i] = reinterpret_cast<const u32x4*>(kcur)[i];
+        } else {
+            const u32x4* row = reinterpret_cast<const u32x4*>(kc + static_cast<size_t>(c) * kvd + kvh * D);
+            #pragma unroll
+            for (int i = 0; i < D / 8; ++i) kr[i] = row[i];
+        }
+        float acc = 0.0f;
+        #pragma unroll
+        for (int i = 0; i < D / 8; ++i) {
+            const u32x4 qq = reinterpret_cast<const u32x4*>(qv)[i];
+            const uint32_t qd[4] = {qq.x, qq.y, qq.z, qq.w}, kd[4] = {kr[i].x, kr[i].y, kr[i].z, kr[i].w};
+            #pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc = fmaf(h_f(static_cast<uint16_t>(qd[j] & 0xffffu)), h_f(static_cast<uint16_t>(kd[j] & 0xffffu)), acc);
+                acc = fmaf(h_f(static_cast<uint16_t>(qd[j] >> 16)), h_f(static_cast<uint16_t>(kd[j] >> 16)), acc);
+            }
+        }
+        const float sco = h_f(f_h(acc * scale));
+        sc[c - k0] = sco;
+        m = fmaxf(m, sco);
+    }
+    m = wave_max(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float l = 0.0f;
+    for (int c = k0 + tid; c < k1; c += kSplitThreads) {
+        const float e = exp_poly(sc[c - k0] - m);
+        sc[c - k0] = e;
+        l += e;
+    }
+    for (int sft = 32; sft > 0; sft >>= 1) l += __shfl_xor(l, sft, 64);
+    if (lane == 0) red[4 + wave] = l;
+    __syncthreads();                                           // exponentials and the waves' sums are in LDS
+    // o[d]: kSplitThreads / D groups of D threads, group g takes the keys k0 + g, k0 + g + groups, ...
+    constexpr int kGroups = kSplitThreads / D;
+    const int d = tid % D, grp = tid / D;
+    float o = 0.0f;
+    #pragma unroll 8
+    for (int c = k0 + grp; c < k1; c += kGroups) {
+        const uint16_t v = c == pos ? vcur[d] : vc[static_cast<size_t>(c) * kvd + kvh * D + d];
+        o = fmaf(sc[c - k0], h_f(v), o);
+    }
+    osum[grp * D + d] = o;
+    __syncthreads();
+    if (tid < D) {
+        float t = osum[tid];
+        #pragma unroll
+        for (int g2 = 1; g2 < kGroups; ++g2) t += osum[g2 * D + tid];
+        mine[2 + tid] = t;
+    }
+    if (tid == 0) {
+        mine[0] = m;
+        mine[1] = (red[4] + red[5]) + (red[6] + red[7]);
+    }
+}
+
+// The parts of a head into its attention output (see attention_split_kernel).  Every load of the launch is
+// asked for before the first is used: thread s takes the maximum and the sum of part s, thread d element d
+// of every part.
+template <int D>
+__global__ __launch_bounds__(D) void attention_merge_kernel(const float* __restrict__ part, int splits,
+                                                            uint16_t* __restrict__ out) {
+    __shared__ float w[kMaxSplits];
+    __shared__ float Ls;
+    const int qh = blockIdx.x, d = threadIdx.x;
+    const float* p = part + static_cast<size_t>(qh) * splits * (D + 2);
+    float o_s[kMaxSplits];
+    #pragma unroll
+    for (int s = 0; s < kMaxSplits; ++s) o_s[s] = s < splits ? p[s * (D + 2) + 2 + d] : 0.0f;
+    if (d < 64) {                                              // the first wavefront: splits <= 32 lanes of it
+        const bool has = d < splits;
+        const float ms = has ? p[d * (D + 2)] : -3.402823466e+38f;
+        const float ls = has ? p[d * (D + 2) + 1] : 0.0f;
+        const float M = wave_max(ms);
+        const float ws = ls > 0.0f ? exp_poly(ms - M) : 0.0f;
+        float L = ls * ws;
+        for (int sft = 32; sft > 0; sft >>= 1) L += __shfl_xor(L, sft, 64);
+        if (d < kMaxSplits) w[d] = ws;
+        if (d == 0) Ls = L;
+    }
+    __syncthreads();
+    float o = 0.0f;
+    #pragma unroll
+    for (int s = 0; s < kMaxSplits; ++s) o = fmaf(o_s[s], w[s], o);
+    out[qh * D + d] = f_h(o * rcp_rn(Ls + 1e-20f));
+}
+
+inline size_t split_attention_lds(int D, int chunk_cap) {
+    return static_cast<size_t>(chunk_cap + 8 + kSplitThreads) * 4 + 3 * static_cast<size_t>(D) * 2;
+}
+
 // gate[i] = fp16((g * sigmoid(g)) * up[i])   (QW/kernels/mlp.cl swiglu_inplace)
 __global__ void swiglu_kernel(uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, int n) {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
@@ -1000,6 +1174,9 @@ struct Decoder {
     // or two.  An entry stays null where a layer's matrices are not of one kind.
     std::vector<void*> wqkv, wgu, stacked_mem;
     bool stacked_built = false;
+    // attention with a head's keys split over blocks (mi_decoder_set_attention_splits): 0 = the reference-order launch
+    int splits = 0;
+    float* split_part = nullptr;                               // [n_heads][splits][head_dim + 2]
 };
 
 template <typename T>
@@ -1144,6 +1321,21 @@ int mi_decoder_read(void* dec, void* stream, int* pos, int* token) {
 
 const void* mi_decoder_logits(void* dec) { return dec ? static_cast<Decoder*>(dec)->logits : nullptr; }
 
+int mi_decoder_set_attention_splits(void* dec, int splits) {
+    auto* d = static_cast<Decoder*>(dec);
+    if (!d) return 0;
+    if (splits <= 1) { d->splits = 0; return 1; }
+    const int D = d->c.head_dim;
+    if (splits > kMaxSplits || (D != 64 && D != 128)) {
+        MI_ERROR_FMT("mi_decoder_set_attention_splits: %d splits at head_dim %d (2..%d, head_dim 64 or 128)", splits, D, kMaxSplits);
+        return 0;
+    }
+    if (!d->split_part &&
+        !dev_alloc(d, &d->split_part, static_cast<size_t>(d->c.n_heads) * kMaxSplits * (D + 2) * sizeof(float))) return 0;
+    d->splits = splits;
+    return 1;
+}
+
 const void* mi_decoder_buffer(void* dec, int which) {
     auto* d = static_cast<Decoder*>(dec);
     if (!d) return nullptr;
@@ -1266,7 +1458,22 @@ int mi_decoder_step(void* dec, void* stream) {
         uint16_t* vc = d->vc + static_cast<size_t>(l) * c.max_pos * kvd;
         const auto *bq = static_cast<const uint16_t*>(d->bq[l]), *bk = static_cast<const uint16_t*>(d->bk[l]),
                    *bv = static_cast<const uint16_t*>(d->bv[l]);
-        if (D == 64 || D == 128) {
+        if (d->splits > 1) {
+            const int chunk_cap = ((c.max_pos + d->splits - 1) / d->splits + 3) & ~3;
+            const size_t lds = split_attention_lds(D, chunk_cap);
+            const dim3 grid(c.n_heads, d->splits);
+            if (D == 64) {
+                hipLaunchKernelGGL(attention_split_kernel<64>, grid, dim3(kSplitThreads), lds, s, kc, vc, d->st, c.n_heads,
+                                   c.n_kv_heads, c.max_pos, scale, d->q, d->k, d->v, bq, bk, bv, d->rope_now, d->qr, d->kr,
+                                   d->vr, d->split_part, chunk_cap);
+                hipLaunchKernelGGL(attention_merge_kernel<64>, dim3(c.n_heads), dim3(64), 0, s, d->split_part, d->splits, d->attn);
+            } else {
+                hipLaunchKernelGGL(attention_split_kernel<128>, grid, dim3(kSplitThreads), lds, s, kc, vc, d->st, c.n_heads,
+                                   c.n_kv_heads, c.max_pos, scale, d->q, d->k, d->v, bq, bk, bv, d->rope_now, d->qr, d->kr,
+                                   d->vr, d->split_part, chunk_cap);
+                hipLaunchKernelGGL(attention_merge_kernel<128>, dim3(c.n_heads), dim3(128), 0, s, d->split_part, d->splits, d->attn);
+            }
+        } else if (D == 64 || D == 128) {
             const size_t lds = tiled_attention_lds(D, c.max_pos);
             if (D == 64)
                 hipLaunchKernelGGL(rope_attention_tiled<64>, dim3(c.n_heads), dim3(256), lds, s, kc, vc, d->st, c.n_heads,

@@ -479,6 +479,28 @@ def main():
             detail[f"c5_whole_prompt_on_device_M{M}"] = {
                 "ms": round(ms, 3), "prompt_tokens_per_s": round(M / ms * 1e3, 0),
                 "vs_single_token_steps": round(M * ms_tok / ms, 1)}
+        # a decode step at a long context (positions 1900..1931 of the same decoder; the cache's contents do
+        # not matter for the time): the reference-order attention and the mode that splits a head's keys
+        long_ctx = {"positions": "1900..1931"}
+        for name, splits in (("us_per_token_reference_order", 0), ("us_per_token_16_key_splits", 16)):
+            assert big.set_attention_splits(splits)
+            assert big.reset(queue, 1900, 5) and big.step(queue)
+            queue.finish()
+            assert big.reset(queue, 1900, 5)
+            with mil.Graph(queue) as g:
+                assert big.step(queue)
+
+            def run32():
+                for _ in range(32):
+                    g.launch()
+            samples = []
+            for _ in range(3):
+                assert big.reset(queue, 1900, 5)
+                queue.finish()
+                samples.append(time_region(mil, queue, run32, 1, 1) / 32)
+            long_ctx[name] = round(sorted(samples)[1] * 1e3, 1)
+        assert big.set_attention_splits(0)
+        detail["c4_decode_step_long_context"] = long_ctx
         big.close()
 
     # ---- CPU baseline: the oracle on a bounded sample of the same sweep -------------------

@@ -91,6 +91,16 @@ int   mi_decoder_reserve_prompt(void* decoder, void* stream, int max_tokens);
 /* Reads the device state back (synchronises the stream). */
 int   mi_decoder_read(void* decoder, void* stream, int* pos, int* token);
 /* fp16 [vocab] logits of the last step, in device memory. */
+/* An arithmetic mode of the attention inside mi_decoder_step, for long contexts.  0 or 1 (default): the
+ * launch that keeps the reference's order of operations (QW/kernels/attention.cl: one work-group per
+ * head, the sum of the exponentials and every output element's sum over the keys in key order), bit
+ * for bit; its time grows by about 24 ns per position and layer.  2..32: the keys of a head are taken
+ * by that many blocks, each with its own maximum and sums, and a second launch merges them: the same
+ * real numbers summed in another order, without the fp16 roundings of the probabilities, within
+ * max-abs/rel 1e-3 and cosine 0.9999 of the default, not bit-identical; one launch more per layer.
+ * head_dim 64 or 128.  Allocates once; call it between steps, never under graph capture (a graph
+ * captured afterwards keeps the mode it was captured in).  No counterpart in the reference. */
+int   mi_decoder_set_attention_splits(void* decoder, int splits);
 const void* mi_decoder_logits(void* decoder);
 /* Activations left by the last step, fp16 in device memory, for comparing implementations buffer
  * by buffer: which = 0 residual stream [hidden], 1 q after bias and rotary [n_heads*head_dim],
