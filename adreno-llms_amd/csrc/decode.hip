@@ -561,6 +561,27 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
         return;
     }
     const bool has_current = k1 == seq_k;                      // the block whose run ends with the current position
+    // Everything the block reads from memory is asked for now, behind the position alone: the row of the
+    // thread's first key, the first kAhead values of the thread's output element, and (below) the current
+    // position's q, k and v; the arithmetic then waits for one round trip, not for four in a row.
+    constexpr int kGroups = kSplitThreads / D, kAhead = 32;
+    const int d = tid % D, grp = tid / D;
+    const int c_first = k0 + tid;
+    u32x4 kr_first[D / 8];
+    // (a thread without such a key reads row 0 instead and does not use it: loads under a condition of
+    //  their own were measured slower, 548 -> 576 us per step at position 2000)
+    {
+        const bool from_cache = c_first < k1 && c_first != pos;
+        const u32x4* row = reinterpret_cast<const u32x4*>(kc + static_cast<size_t>(from_cache ? c_first : 0) * kvd + kvh * D);
+        #pragma unroll
+        for (int i = 0; i < D / 8; ++i) kr_first[i] = row[i];
+    }
+    uint16_t v_first[kAhead];
+    #pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+        const int c = k0 + grp + i * kGroups;
+        v_first[i] = vc[static_cast<size_t>(c < k1 && c != pos ? c : 0) * kvd + kvh * D + d];
+    }
     // q of the head (every block), k and v of the current position (the block that needs them); the block of
     // the group's first head also writes them to the caches and to the buffers a caller may inspect
     if (tid < hd2) {
@@ -596,11 +617,14 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
     __syncthreads();
     // scores, a thread per key: the key's row straight from the cache (the current position's from LDS)
     float m = -3.402823466e+38f;
-    for (int c = k0 + tid; c < k1; c += kSplitThreads) {
+    for (int c = c_first; c < k1; c += kSplitThreads) {
         u32x4 kr[D / 8];
         if (c == pos) {
             #pragma unroll
             for (int i = 0; i < D / 8; ++i) kr[i] = reinterpret_cast<const u32x4*>(kcur)[i];
+        } else if (c == c_first) {
+            #pragma unroll
+            for (int i = 0; i < D / 8; ++i) kr[i] = kr_first[i];
         } else {
             const u32x4* row = reinterpret_cast<const u32x4*>(kc + static_cast<size_t>(c) * kvd + kvh * D);
             #pragma unroll
@@ -635,11 +659,14 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
     if (lane == 0) red[4 + wave] = l;
     __syncthreads();                                           // exponentials and the waves' sums are in LDS
     // o[d]: kSplitThreads / D groups of D threads, group g takes the keys k0 + g, k0 + g + groups, ...
-    constexpr int kGroups = kSplitThreads / D;
-    const int d = tid % D, grp = tid / D;
     float o = 0.0f;
+    #pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+        const int c = k0 + grp + i * kGroups;
+        if (c < k1) o = fmaf(sc[c - k0], h_f(c == pos ? vcur[d] : v_first[i]), o);
+    }
     #pragma unroll 8
-    for (int c = k0 + grp; c < k1; c += kGroups) {
+    for (int c = k0 + grp + kAhead * kGroups; c < k1; c += kGroups) {
         const uint16_t v = c == pos ? vcur[d] : vc[static_cast<size_t>(c) * kvd + kvh * D + d];
         o = fmaf(sc[c - k0], h_f(v), o);
     }
