@@ -98,7 +98,9 @@ int   mi_decoder_read(void* decoder, void* stream, int* pos, int* token);
  * by that many blocks, each with its own maximum and sums, and a second launch merges them: the same
  * real numbers summed in another order, without the fp16 roundings of the probabilities, within
  * max-abs/rel 1e-3 and cosine 0.9999 of the default, not bit-identical; one launch more per layer.
- * head_dim 64 or 128.  Allocates once; call it between steps, never under graph capture (a graph
+ * head_dim 64 or 128.  Measured on Qwen2.5-0.5B shapes: 16 is the fastest up to about 2000 positions, 32 beyond
+ * (position 4000: 594 us per step against 659 with 16 and 2723 in the reference's order); below about 150
+ * positions the default is faster.  Allocates once; call it between steps, never under graph capture (a graph
  * captured afterwards keeps the mode it was captured in).  No counterpart in the reference. */
 int   mi_decoder_set_attention_splits(void* decoder, int splits);
 const void* mi_decoder_logits(void* decoder);
