@@ -521,8 +521,8 @@ __global__ __launch_bounds__(256) void rope_attention_tiled(uint16_t* __restrict
 // ---- attention with the keys of a head split over several blocks (an arithmetic mode, not the default) ----
 //
 // The launch above keeps the reference's order of operations, and at a long context that order is two
-// chains of dependent additions as long as the context, in one wavefront per head.  Here block (head, s) of
-// `splits` takes every splits-th run of the keys: scores as above (fp32 dot product, rounded to fp16 like
+// chains of dependent additions as long as the context, in one wavefront per head.  Here block (head, s) takes
+// run s of `splits` consecutive runs of the keys: scores as above (fp32 dot product, rounded to fp16 like
 // the reference's), its own maximum m, e = exp(score - m) in fp32, their sum l and o[d] = sum e v[d]; a
 // second launch merges the parts of a head: M = max m, out = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s.
 // The same real numbers as softmax(q k) v, summed in another order and without the fp16 roundings of the
