@@ -34,6 +34,7 @@ struct Tensor {
     std::vector<int64_t> shape;
     std::string dtype;
     void* dev = nullptr;
+    bool registered = false;
 };
 
 struct Bundle {
@@ -213,7 +214,12 @@ void* mi_bundle_open(const char* bin_path, const char* meta_path) {
 void mi_bundle_close(void* h) {
     auto* b = static_cast<Bundle*>(h);
     if (!b) return;
-    for (auto& kv : b->tensors) if (kv.second.dev) mi_free(kv.second.dev);
+    // registry entries are keyed by the device pointer: they go before the allocation does, so
+    // that a later allocation at the same address is not mistaken for this bundle's weight
+    for (auto& kv : b->tensors) {
+        if (kv.second.registered) mi_unregister_weight(kv.second.dev);
+        if (kv.second.dev) mi_free(kv.second.dev);
+    }
     if (b->map) munmap(const_cast<uint8_t*>(b->map), b->map_size);
     if (b->fd >= 0) close(b->fd);
     delete b;
@@ -258,18 +264,22 @@ int mi_bundle_upload(void* h) {
     // LFM2-VL bundles spell the sibling ".scales" (LV/scripts/quantize_int8.py:91-97).
     int registered = 0;
     for (auto& kv : b->tensors) {
-        const Tensor& t = kv.second;
+        Tensor& t = kv.second;
+        if (t.registered) { ++registered; continue; }
         if ((t.dtype != "int8" && t.dtype != "q4_packed") || t.shape.size() != 2) continue;
         auto sit = b->tensors.find(kv.first + ".scale");
         if (sit == b->tensors.end()) sit = b->tensors.find(kv.first + ".scales");
         if (sit == b->tensors.end()) continue;
         const Tensor& s = sit->second;
+        int ok;
         if (t.dtype == "int8") {
-            registered += mi_register_int8_weight(t.dev, s.dev, static_cast<int>(t.shape[0]), static_cast<int>(t.shape[1]));
+            ok = mi_register_int8_weight(t.dev, s.dev, static_cast<int>(t.shape[0]), static_cast<int>(t.shape[1]));
         } else {
             if (s.shape.size() != 2) continue;
-            registered += mi_register_q4_weight(t.dev, s.dev, static_cast<int>(t.shape[0]), static_cast<int>(s.shape[1] * 32));
+            ok = mi_register_q4_weight(t.dev, s.dev, static_cast<int>(t.shape[0]), static_cast<int>(s.shape[1] * 32));
         }
+        t.registered = ok != 0;
+        registered += ok;
     }
     return registered;
 }

@@ -37,6 +37,8 @@ struct DeviceInfo {
     char arch[64] = {0};
 };
 const DeviceInfo& device_info();
+// First call of any entry point: mi_init(0) unless mi_init has run; safe from several host threads.
+bool ensure_init();
 // 0 = every GEMV evaluates the reference kernels' sum in their order (bit-exact);
 // 1 = Q4 may use the throughput kernel (same fp32 sum, other order).
 // Both are looked up for the stream a call is enqueued on: the value mi_stream_set_modes gave that

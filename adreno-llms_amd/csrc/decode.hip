@@ -1225,7 +1225,7 @@ using namespace mi;
 extern "C" {
 
 void* mi_decoder_create(const mi_decoder_config* cfg, const mi_decoder_weights* w) {
-    if (!cfg || !w || mi_init(0) != 1) return nullptr;
+    if (!cfg || !w || !ensure_init()) return nullptr;
     const mi_decoder_config& c = *cfg;
     if (c.hidden <= 0 || c.inter <= 0 || c.n_heads <= 0 || c.n_kv_heads <= 0 || c.head_dim <= 0 || c.n_layers <= 0 ||
         c.vocab <= 0 || c.max_pos <= 0 || c.n_heads % c.n_kv_heads || c.head_dim % 4 || c.head_dim > 256 || c.max_pos > kMaxPositions) {

@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const u32x4* __restric
 
 extern "C" int mi_stream_read_probe(void* stream, const void* src, size_t bytes, void* sink) {
     using namespace mi;
-    if (mi_init(device_info().device < 0 ? 0 : device_info().device) != 1) return 0;
+    if (!ensure_init()) return 0;
     if (!src || bytes < 16 || reinterpret_cast<uintptr_t>(src) % 16) {
         MI_ERROR_FMT("mi_stream_read_probe: bad argument (src=%p bytes=%zu)", src, bytes);
         return 0;

@@ -17,8 +17,11 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 namespace mi {
 namespace {
 
+// Written by mi_init under g_init_mu; every other entry point reads them only after it has seen
+// g_inited true (acquire), so host threads that arrive together at a first call initialise once.
 DeviceInfo g_dev;
-bool g_inited = false;
+std::atomic<bool> g_inited{false};
+std::mutex g_init_mu;
 // Process defaults of the two arithmetic modes; a stream can carry its own (mi_stream_set_modes),
 // so that host threads driving different streams do not change each other's arithmetic.
 std::atomic<int> g_gemm_mode{0};
@@ -67,11 +70,6 @@ void add_workspace(hipStream_t s) {
     g_workspace[s] = p;
 }
 
-bool ensure_init() {
-    if (g_inited) return true;
-    return mi_init(0) == 1;
-}
-
 bool lookup(const void* W, Entry* out) {
     std::lock_guard<std::mutex> lk(g_registry_mu);
     auto it = g_registry.find(W);
@@ -99,6 +97,11 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 }  // namespace
 
 const DeviceInfo& device_info() { return g_dev; }
+
+bool ensure_init() {
+    if (g_inited.load(std::memory_order_acquire)) return true;
+    return mi_init(0) == 1;
+}
 
 bool registered_weight(const void* W, int N, int K, WeightKind* kind, const void** scale) {
     Entry e;
@@ -184,6 +187,7 @@ using namespace mi;
 extern "C" {
 
 int mi_init(int device) {
+    std::lock_guard<std::mutex> init_lk(g_init_mu);
     int count = 0;
     if (!MI_HIP_OK(hipGetDeviceCount(&count))) return 0;
     if (device < 0 || device >= count) {
@@ -207,8 +211,8 @@ int mi_init(int device) {
     g_dev.device = device;
     g_dev.cus = prop.multiProcessorCount;
     std::snprintf(g_dev.arch, sizeof(g_dev.arch), "%s", prop.gcnArchName);
-    if (!g_inited && !workspace_of(nullptr)) add_workspace(nullptr);      // the null stream's GEMM workspace
-    g_inited = true;
+    if (!workspace_of(nullptr)) add_workspace(nullptr);      // the null stream's GEMM workspace
+    g_inited.store(true, std::memory_order_release);
     return 1;
 }
 
@@ -418,7 +422,7 @@ int mi_linear_argmax(void* stream, int N, int K, const void* x, const void* W, v
 int mi_linear_argmax_static(void* stream, int N, int K, const void* x, const void* W, void* logits, int num_partials,
                             void* token_out) {
     // (no lazy set-up here: mi_init allocates the null stream's workspace, and this entry point allocates nothing)
-    if (!g_inited) {
+    if (!g_inited.load(std::memory_order_acquire)) {
         MI_ERROR_FMT("mi_linear_argmax_static: mi_init has not run on this process");
         return 0;
     }
@@ -513,6 +517,13 @@ int mi_linear_batch(void* stream, const mi_linear_call* calls, int n) {
     return n;
 }
 
+// An executable graph remembers the stream it was recorded on: the launches inside it use that
+// stream's workspace (K slices of a GEMM, argmax candidates), which only that stream's order protects.
+struct RecordedGraph {
+    hipGraphExec_t exec;
+    hipStream_t origin;
+};
+
 int mi_graph_begin(void* stream) {
     if (!ensure_init()) return 0;
     if (!stream) { MI_ERROR_FMT("mi_graph_begin: needs a stream made by mi_stream_create"); return 0; }
@@ -525,16 +536,27 @@ void* mi_graph_end(void* stream) {
     hipGraphExec_t exec = nullptr;
     const bool ok = MI_HIP_OK(hipGraphInstantiate(&exec, g, nullptr, nullptr, 0));
     (void)hipGraphDestroy(g);      // the executable graph keeps what it needs
-    return ok ? exec : nullptr;
+    return ok ? new RecordedGraph{exec, as_stream(stream)} : nullptr;
 }
 
 int mi_graph_launch(void* graph, void* stream) {
     if (!graph) { MI_ERROR_FMT("mi_graph_launch: null graph"); return 0; }
-    return MI_HIP_OK(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), as_stream(stream))) ? 1 : 0;
+    auto* g = static_cast<RecordedGraph*>(graph);
+    if (as_stream(stream) != g->origin) {
+        MI_ERROR_FMT("mi_graph_launch: graph recorded on stream %p launched on stream %p; its launches use the "
+                     "recording stream's workspace, so it replays on that stream only",
+                     static_cast<void*>(g->origin), stream);
+        return 0;
+    }
+    return MI_HIP_OK(hipGraphLaunch(g->exec, g->origin)) ? 1 : 0;
 }
 
 int mi_graph_destroy(void* graph) {
-    return graph ? (MI_HIP_OK(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph))) ? 1 : 0) : 1;
+    if (!graph) return 1;
+    auto* g = static_cast<RecordedGraph*>(graph);
+    const int ok = MI_HIP_OK(hipGraphExecDestroy(g->exec)) ? 1 : 0;
+    delete g;
+    return ok;
 }
 
 int mi_linear_add(void* stream, int M, int N, int K, const void* x, const void* W, void* residual) {

@@ -159,7 +159,10 @@ int mi_linear_batch(void* stream, const mi_linear_call* calls, int n);
 /* Record / replay of everything enqueued on a stream between begin and end, as a HIP graph;
  * the counterpart of the reference's recordable-queue replay of the decode step
  * (NNOPT_RECORD, QW/src/model.cpp:709-720).  Only kernel launches may be recorded: no
- * mi_malloc, mi_memcpy_* or mi_memset between begin and end. */
+ * mi_malloc, mi_memcpy_* or mi_memset between begin and end.  A graph replays on the stream it
+ * was recorded on and on no other: its launches use that stream's workspace (the K slices of a
+ * GEMM, the argmax candidates), which only that stream's order keeps apart from the stream's
+ * other work; mi_graph_launch with another stream prints an error and returns 0. */
 int   mi_graph_begin(void* stream);
 void* mi_graph_end(void* stream);              /* returns an executable graph or NULL */
 int   mi_graph_launch(void* graph, void* stream);

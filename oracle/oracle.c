@@ -268,6 +268,13 @@ int orc_max_threads(void)
 #endif
 }
 
+/* The flags this library was compiled with (oracle/Makefile passes them in), for the benchmark's
+ * CPU-baseline record. */
+#ifndef ORC_BUILD_FLAGS
+#define ORC_BUILD_FLAGS "unknown"
+#endif
+const char* orc_build_flags(void) { return ORC_BUILD_FLAGS; }
+
 static int clamp_threads(int n)
 {
     if (n < 1) n = 1;

@@ -42,6 +42,10 @@
  *        of evaluation order: the reference's device code is built with
  *        -cl-fast-relaxed-math and holds no known-answer vector for a GEMV, so
  *        there is no reference bit pattern to match.
+ *   orc_gemv_q4_add : the reference has no Q4 residual kernel (its fused residual form,
+ *        SM/kernels/block_fused_int8.cl:105-174, is int8 only), so the mathematics pins it:
+ *        res + dequant(W) x in fp64 within one fp16 step, zero residual == orc_gemv_q4
+ *        bit for bit, a swamping residual returned unchanged (tests/test_oracle_gemv.py).
  *   decode.c (rmsnorm, rotary, attention, SwiGLU, adds, whole step): fp64
  *        statements and index probes in tests/test_oracle_decode.py.
  */
@@ -97,6 +101,7 @@ void orc_gemm_i8 (const uint16_t* X, const int8_t* q, const uint16_t* s, uint16_
 void orc_gemm_q4 (const uint16_t* X, const uint8_t* p, const uint16_t* sc, uint16_t* out, int M, int N, int K, int n_threads);
 
 int orc_max_threads(void);
+const char* orc_build_flags(void);   /* compiler and flags of this build */
 
 /* argmax_partial (NP work-groups of 64 over contiguous chunks) + argmax_finalize, literally:
  * QW/kernels/gemv_m1.cl:198-280.  Index of the greatest fp16 value with the kernels' own tie

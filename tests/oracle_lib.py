@@ -49,6 +49,7 @@ def _load():
         "orc_gemm_i8": (None, [_u16p, _i8p, _u16p, _u16p, I, I, I, I]),
         "orc_gemm_q4": (None, [_u16p, _u8p, _u16p, _u16p, I, I, I, I]),
         "orc_max_threads": (I, []),
+        "orc_build_flags": (C.c_char_p, []),
         "orc_argmax_f16": (I, [_u16p, I, I]),
     }
     for name, (res, args) in sig.items():

@@ -38,7 +38,14 @@ def test_json_line_has_the_contract_keys():
         assert key in rf, key
     assert rf["bound"] == "hbm" and rf["peak"] == 8000.0 and rf["unit"] == "GB/s"
     assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-3 and 0.3 < rf["frac"] < 1.0
+    # the launch the step's time goes to, beside the launch its bytes go to, and the step itself
+    bt = rf["by_time"]
+    for key in ("kernel", "bound", "achieved", "peak", "unit", "frac", "share_of_step", "us_per_launch", "bytes_per_launch"):
+        assert key in bt, key
+    assert 0.0 < bt["frac"] < 1.0 and 0.0 < bt["share_of_step"] <= 1.0
+    assert abs(rf["step"]["frac"] - d["value"] / 8000.0) < 1e-3
     cb = d["cpu_baseline"]
+    assert "-O3" in cb["compiler_flags"]
     for key in ("value", "unit", "cores", "kind", "sample"):
         assert key in cb, key
     assert cb["kind"] in ("port", "reference") and cb["cores"] >= 1 and cb["value"] > 0

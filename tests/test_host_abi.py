@@ -85,3 +85,71 @@ int main(void) {
     assert r.returncode == 0, r.stderr
     r = subprocess.run([str(exe)], capture_output=True, text=True)
     assert r.returncode == 0 and r.stdout.startswith("ok"), (r.returncode, r.stdout, r.stderr)
+
+
+THREADS_PROGRAM = r'''
+#include "mi_linear.h"
+#include <pthread.h>
+#include <stdint.h>
+#include <stdio.h>
+/* Host threads on the registry and the per-stream modes at once: each thread registers, looks up,
+ * re-registers and unregisters its own keys and sets modes for its own stream handles, while all of
+ * them also hammer a few shared keys.  The calls touch no device. */
+enum { THREADS = 4, KEYS = 2000, ROUNDS = 20 };
+static void* work(void* arg) {
+    uintptr_t t = (uintptr_t)arg;
+    long bad = 0;
+    for (int r = 0; r < ROUNDS; ++r) {
+        for (uintptr_t i = 1; i <= KEYS; ++i) {
+            const void* mine = (const void*)((t + 1) * 0x1000000u + i * 64);
+            const void* shared = (const void*)(0x900000u + (i % 7) * 64);
+            bad += mi_register_int8_weight(mine, (const void*)0x10, 8, 64) != 1;
+            bad += mi_weight_kind(mine) != 8;
+            bad += mi_register_q4_weight(mine, (const void*)0x10, 8, 64) != 1;
+            bad += mi_weight_kind(mine) != 4;
+            mi_register_int8_weight(shared, (const void*)0x10, 4, 32);
+            int k = mi_weight_kind(shared);
+            bad += !(k == 8 || k == 0);
+            mi_unregister_weight(shared);
+            bad += mi_stream_set_modes((void*)mine, (int)(i & 1), 1) != 1;
+            if (r + 1 < ROUNDS || (i & 3)) {
+                bad += mi_unregister_weight(mine) != 1;
+                bad += mi_weight_kind(mine) != 0;
+                bad += mi_stream_set_modes((void*)mine, -1, -1) != 1;
+            }
+        }
+    }
+    return (void*)bad;
+}
+int main(void) {
+    pthread_t th[THREADS];
+    long bad = 0;
+    for (uintptr_t t = 0; t < THREADS; ++t) pthread_create(&th[t], 0, work, (void*)t);
+    for (int t = 0; t < THREADS; ++t) { void* r; pthread_join(th[t], &r); bad += (long)r; }
+    long left = 0;
+    for (uintptr_t t = 0; t < THREADS; ++t)
+        for (uintptr_t i = 1; i <= KEYS; ++i) {
+            const void* mine = (const void*)((t + 1) * 0x1000000u + i * 64);
+            int k = mi_weight_kind(mine);
+            if (i & 3) bad += k != 0; else { bad += k != 4; ++left; mi_unregister_weight(mine); }
+        }
+    printf("bad %ld left %ld\n", bad, left);
+    return bad != 0;
+}
+'''
+
+
+def test_host_threads_share_the_registry_and_the_stream_modes(tmp_path):
+    """The reference's host is single threaded (QW/src/utils.cpp:63-66: plain statics); this library's
+    registry and per-stream modes sit behind a mutex, which four threads exercise here without a GPU."""
+    import subprocess
+    src = tmp_path / "threads.c"
+    src.write_text(THREADS_PROGRAM)
+    exe = tmp_path / "threads"
+    libdir = os.path.dirname(mil.LIB_PATH)
+    cmd = ["gcc", "-std=c11", "-O1", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+           "-L", libdir, "-lmi_linear", f"-Wl,-rpath,{libdir}", "-lpthread"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.strip() == "bad 0 left 2000", (r.returncode, r.stdout, r.stderr[-2000:])

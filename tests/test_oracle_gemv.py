@@ -285,3 +285,41 @@ def test_threads_do_not_change_bits():
     W, x = _rand(64, 896, 20)
     q, s = O.quantize_int8(W)
     assert np.array_equal(O.gemv_i8(x, q, s, threads=1), O.gemv_i8(x, q, s, threads=O.THREADS))
+
+
+@pytest.mark.parametrize("N,K", [(24, 1024), (16, 896), (5, 4864), (7, 96)])
+def test_q4_residual_add_epilogue(N, K):
+    """orc_gemv_q4_add: the reference has an int8 residual kernel only (SM/kernels/block_fused_int8.cl:105-174),
+    so the mathematics pins the Q4 form: res + dequant(W) x in float64 within one fp16 step (a subtracted or
+    dropped residual, a residual added after the rounding of the product, a wrong row's residual all fail:
+    the residuals are large against the products and differ per row), a zero residual gives orc_gemv_q4's
+    bits (x + 0 is x in fp32), and a residual that swamps the product comes back unchanged."""
+    rng = np.random.default_rng(31 + K)
+    W, x = _rand(N, K, 32 + N)
+    p, sc = O.quantize_q4(W)
+    sc = np.ascontiguousarray(sc)
+    xs = O.u16(x)
+    wf = np.empty((N, K), np.float32)
+    O.lib.orc_dequant_q4_to_f32(p, sc, N, K, wf)
+    prod = wf.astype(np.float64) @ x.astype(np.float64)
+
+    res0 = (rng.standard_normal(N) * 3 + np.arange(N)).astype(np.float16)
+    res = O.u16(res0).copy()
+    O.lib.orc_gemv_q4_add(xs, p, sc, res, N, K)
+    want = prod + res0.astype(np.float64)
+    got = O.f16(res).astype(np.float64)
+    # one fp16 step at the result's size (2^-10 relative), plus the fp32 accumulation error of the sum
+    assert np.all(np.abs(got - want) <= np.abs(want) * 2.0**-10 + 1e-5)
+    # the tolerance separates it from the two-rounding form only on average, so also: most outputs are
+    # the correctly rounded fp16 of the fp64 value
+    exact = want.astype(np.float16).astype(np.float64)
+    assert np.mean(got == exact) >= 0.9
+
+    zero = np.zeros(N, np.uint16)
+    O.lib.orc_gemv_q4_add(xs, p, sc, zero, N, K)
+    assert np.array_equal(zero, O.gemv_q4(x, p, sc))
+
+    big = O.u16(np.full(N, 60000.0, np.float16)).copy()
+    O.lib.orc_gemv_q4_add(xs, p, sc, big, N, K)
+    assert np.all(np.abs(O.f16(big).astype(np.float64) - (60000.0 + prod)) <= 32.0)   # one fp16 step at 6e4
+    assert np.all(np.isfinite(O.f16(big)))
