@@ -1369,7 +1369,10 @@ double gemm_estimate_us(WeightKind kind, int M, int N, int K, size_t workspace_b
 
 GemmPlan plan_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, size_t workspace_bytes) {
     GemmPlan p;
-    const int mode = gemm_mode(s) == 4 && kind != WK_Q4 ? 0 : gemm_mode(s);   // mode 4 only concerns Q4 weights
+    int mode = gemm_mode(s) == 4 && kind != WK_Q4 ? 0 : gemm_mode(s);   // mode 4 only concerns Q4 weights
+    // 100 s + 10 + t: the wide kernel pinned to 32 t rows of x per block and s slices of K
+    int pin_splits = 0;
+    if (mode >= 111) { pin_splits = mode / 100; mode %= 100; }
     const int cus = device_info().cus;
     const bool wide_fits = wide_reaches(kind, M, N, K);
     int tm = 1, splits = 1;
@@ -1390,6 +1393,7 @@ GemmPlan plan_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, size_t w
         const bool may_slice = mode == 0 || mode == 4;
         wide::pick_shape(WK_Q4, p.terms, M, N, K, cus, may_slice ? workspace_bytes : 0, &tm, &splits, nullptr);
         if (mode >= 11 && mode <= 15) tm = mode - 10;
+        if (pin_splits) splits = pin_splits;
         p.kernel = 1; p.tile_rows = 32 * tm; p.k_slices = splits;
         return p;
     }
@@ -1406,6 +1410,7 @@ GemmPlan plan_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, size_t w
         // modes 3 and 11..15 pin the plain kernel; slices of K are the library's own choice (mode 0)
         wide::pick_shape(kind, 1, M, N, K, cus, mode == 0 ? workspace_bytes : 0, &tm, &splits, &wide_us);
         if (mode >= 11) tm = mode - 10;
+        if (pin_splits) splits = pin_splits;
         if (mode != 0 || wide_us < tiled_estimate_us(M, N, K)) {
             p.kernel = 1; p.tile_rows = 32 * tm; p.k_slices = splits;
             return p;

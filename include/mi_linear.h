@@ -177,7 +177,8 @@ int   mi_graph_destroy(void* graph);
  * 2, 3 and 11..15 = as 0 with the kernel choice pinned (tests and tuning: results stay within
  * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel (int8 and fp16
  * weights; fails for Q4), 3 = the wide kernel, 10 + t (t = 1..5) = the wide kernel with 32 t
- * rows of x per block, 5 = the streaming kernel for up to 64 rows of x (every kind of weights takes
+ * rows of x per block, 100 s + 10 + t (s = 1..24) = the same with K cut into s slices (refused where the
+ * slices' fp32 sums do not fit the stream's workspace), 5 = the streaming kernel for up to 64 rows of x (every kind of weights takes
  * it by itself in mode 0 up to 32 to 64 rows, depending on the shape, where it is the faster one;
  * fails for more than 64 rows).
  * Q4 weights: a weight q * scale (4 and 11 significant bits) is not an fp16 number in general.
