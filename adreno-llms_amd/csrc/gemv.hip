@@ -1279,7 +1279,7 @@ bool launch_gemv_group(hipStream_t s, const GemvCall* calls, int n) {
     if (c.epi == EPI_SWIGLU) {
         if (n != 2 || calls[0].N != calls[1].N || c.M != 1 || !gemv_takes_swiglu(c.kind, c.K)) {
             MI_ERROR_FMT("gemv: the SwiGLU epilogue takes a gate and an up matrix of equal N, M = 1 "
-                         "and K in {576, 896, 1024, 1536} (n=%d kind=%d K=%d)", n, static_cast<int>(c.kind), c.K);
+                         "and K in {576, 896, 960, 1024, 1536, 2048} (n=%d kind=%d K=%d)", n, static_cast<int>(c.kind), c.K);
             return false;
         }
         if (c.kind == WK_I8) {

@@ -90,7 +90,6 @@ int   mi_decoder_reserve_prompt(void* decoder, void* stream, int max_tokens);
 
 /* Reads the device state back (synchronises the stream). */
 int   mi_decoder_read(void* decoder, void* stream, int* pos, int* token);
-/* fp16 [vocab] logits of the last step, in device memory. */
 /* An arithmetic mode of the attention inside mi_decoder_step, for long contexts.  0 or 1 (default): the
  * launch that keeps the reference's order of operations (QW/kernels/attention.cl: one work-group per
  * head, the sum of the exponentials and every output element's sum over the keys in key order), bit
@@ -103,6 +102,7 @@ int   mi_decoder_read(void* decoder, void* stream, int* pos, int* token);
  * positions the default is faster.  Allocates once; call it between steps, never under graph capture (a graph
  * captured afterwards keeps the mode it was captured in).  No counterpart in the reference. */
 int   mi_decoder_set_attention_splits(void* decoder, int splits);
+/* fp16 [vocab] logits of the last step, in device memory. */
 const void* mi_decoder_logits(void* decoder);
 /* Activations left by the last step, fp16 in device memory, for comparing implementations buffer
  * by buffer: which = 0 residual stream [hidden], 1 q after bias and rotary [n_heads*head_dim],

@@ -40,9 +40,9 @@ def _run(queue, N, K, x, p, sc, add_to=None):
 
 
 @pytest.mark.parametrize("N,K", [(4864, 896), (151936, 896), (4608, 1024), (8192, 576), (4100, 1536), (4099, 896),
-                                 (8192, 2048), (4101, 2048), (4100, 2560), (49152, 960),
+                                 (8192, 2048), (4101, 2048), (4100, 2560), (49152, 960), (4100, 960),
                                  # K values without an instance of their own: the same arithmetic with x in LDS
-                                 (4100, 960), (4099, 1280), (4096, 3072), (4098, 4096), (4096, 8192), (4097, 11008),
+                                 (4099, 1280), (4096, 3072), (4098, 4096), (4096, 8192), (4097, 11008),
                                  (4096, 32), (4100, 30720)])
 def test_fast_q4_within_tolerance(queue, N, K):
     print(f"fast q4 N={N} K={K}", flush=True)
@@ -51,11 +51,17 @@ def test_fast_q4_within_tolerance(queue, N, K):
     got = _run(queue, N, K, x, p, sc)
     want = O.gemv_q4(x, p, sc.view(np.uint16))
     assert_tolerance(got.view(np.float16), want.view(np.float16))
-    # nearly all outputs are the same half (a longer row has more additions whose order differs)
-    assert np.mean(got == want) > (0.96 if K <= 1536 else 0.94 if K <= 2560 else 0.8)
+    same = float(np.mean(got == want))
+    print(f"fast q4 N={N} K={K} identical halves {same:.4f}", flush=True)
+    # Nearly all outputs are the same half.  The others sit next to a rounding boundary, where another order
+    # of the same fp32 additions lands on the other side; a longer row has more additions, and the share grows
+    # about as sqrt(K).  Measured: 0.966 at K = 32, 0.987 at 576, 0.972 at 896, 0.956 at 2560, 0.945 at 8192,
+    # 0.923 at 11 008.  The line below follows those with a margin of 0.01 to 0.03; an error in how the staged x
+    # is paired or ordered moves every output and falls far below it at any K.
+    assert same > 0.96 - 0.0005 * np.sqrt(K)
 
 
-@pytest.mark.parametrize("K", [896, 2048, 2560, 960, 3072, 8192])
+@pytest.mark.parametrize("K", [896, 2048, 2560, 960, 3072, 8192, 11008, 30720])
 def test_fast_q4_exact_on_integer_data_and_all_bytes(queue, K):
     # integer activations and power-of-two scales: every order of the fp32 sum is exact
     rng = np.random.default_rng(5)
@@ -71,13 +77,13 @@ def test_fast_q4_exact_on_integer_data_and_all_bytes(queue, K):
     assert np.array_equal(got, O.gemv_q4(x, p, sc.view(np.uint16)))
 
 
-@pytest.mark.parametrize("K", [896, 1280])
+@pytest.mark.parametrize("K", [896, 1280, 11008])
 def test_fast_q4_unit_vectors_and_subnormal_activations(queue, K):
     N = 4096
     W = synth_w(1200, N, K)
     p, sc = mil.quantize_q4(W)
     nib = np.stack([p & 15, p >> 4], -1).reshape(N, K).astype(np.float32) - 8
-    for k in (0, 1, 4, 5, 31, 32, 511, 512, 895, K - 1):
+    for k in (0, 1, 4, 5, 31, 32, 511, 512, 895, K // 2 + 17, K - 33, K - 1):
         x = np.zeros(K, np.float16)
         x[k] = 1.0
         want = (nib[:, k] * sc[:, k // 32].astype(np.float32)).astype(np.float16)

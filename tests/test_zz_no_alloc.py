@@ -69,10 +69,31 @@ def test_static_scratch_entry_point_matches_the_allocating_one():
                 la, ta, lb, tb = _both(own, stream_handle, sync, c, parts)
                 assert np.array_equal(la, lb), (c["kind"], c["N"])
                 assert ta == tb == O.argmax_f16(la, parts), (c["kind"], c["N"], parts, ta, tb)
-        # beyond the stated maximum: refused before anything is launched
+        # it allocates nothing: every kernel above has run once (its code is loaded), and across further
+        # calls of every path, on both streams, the device's free memory does not move
+        def free_bytes():
+            free, total = ctypes.c_size_t(), ctypes.c_size_t()
+            assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+            return free.value
+        outs = {id(c): (mil.Buffer(c["N"] * 2), mil.Buffer(4)) for c in cases}
+        own.finish()
+        hip.hipStreamSynchronize(foreign)
+        before = free_bytes()
+        for stream_handle, sync in ((foreign, lambda: hip.hipStreamSynchronize(foreign)), (own.handle, own.finish)):
+            for c, parts in ((big, 32), (small, 100), (mid, 1), (q4, 32), (odd, 32)):
+                lb, tb = outs[id(c)]
+                assert mil.lib().mi_linear_argmax_static(stream_handle, c["N"], c["K"], c["x"].ptr, c["W"].ptr, lb.ptr,
+                                                         parts, tb.ptr)
+                assert free_bytes() == before, (c["kind"], c["N"])
+            sync()
+            assert free_bytes() == before
+        # beyond the stated maximum: refused before anything is launched.  W is plain fp16 memory that
+        # no registration describes, so nothing but the limit itself can be what refuses the call.
         too_many = (1 << 22) + 4
         tok = mil.Buffer.from_host(np.array([-7], np.int32))
-        assert mil.lib().mi_linear_argmax_static(own.handle, too_many, 896, big["x"].ptr, big["W"].ptr,
+        plain_w = mil.Buffer(4096)
+        assert mil.lib().mi_weight_kind(plain_w.ptr) == 0
+        assert mil.lib().mi_linear_argmax_static(own.handle, too_many, 896, big["x"].ptr, plain_w.ptr,
                                                  big["W"].ptr, 32, tok.ptr) == 0
         own.finish()
         assert int(tok.read(np.int32, (1,))[0]) == -7
