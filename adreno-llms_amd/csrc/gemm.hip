@@ -797,15 +797,16 @@ inline double estimate_us(int kind, int terms, int tm, int splits, int M, int N,
     //  shapes decides and the general factor holds: 2048 x 896 x 4864 unsliced 47 against 37 us in two slices.
     //  32-row tiles likewise at a K of 1280 to 3072, where the 64 x 64 tiles slow down as soon as a CU holds
     //  two of them: 1536 x 576 x 1536 19.2 -> 14.6 us, 1024 x 2048 x 2048 23.2 -> 18.4, 192 x 8192 x 2048 21.6 ->
-    //  17.3, fp16 1536 x 1024 x 2560 29.6 -> 22.7; at a shorter K the 64 x 64 tiles stay ahead (1536 x 1152 x 896
-    //  10.2 against 11.2), at a longer one slices do (1536 x 896 x 4864 32.6 against 37.7).
+    //  17.3, fp16 1536 x 1024 x 2560 29.6 -> 22.7, and from K = 1024 on (2048 x 1024 x 1024: 12.2 against 14.5 us);
+    //  at a shorter K the 64 x 64 tiles stay ahead (1536 x 1152 x 896 10.2 against 11.2), at a longer one
+    //  slices do (1536 x 896 x 4864 32.6 against 37.7).
     //  Q4 weights in two terms behave the same there (1024 x 2048 x 2048 in 32-row tiles 29.1 us against 34.0
     //  in two slices, 256 x 8192 x 2048 29.2 against 35.0, 2048 x 576 x 1536 21.7 against 24.2), and their tall
     //  tiles, one block per CU and twice the matrix work per byte, lose less to a full chip than the general
     //  factors say: 2048 x 4864 x 896 in 160-row tiles 34.8 us (a block alone: 27.4), 4096 x 8192 x 2048 in
     //  128-row tiles 231 us for four rounds of 48.4, against 258 us for the 64-row tiles the factors preferred.)
     const bool roomy = splits == 1 && blocks > cus / 2 && blocks <= cus &&
-                       (tm == 2 || (tm == 1 && stages >= 20 && stages <= 48));
+                       (tm == 2 || (tm == 1 && stages >= 16 && stages <= 48));
     const bool q4_tall = kind == WK_Q4 && terms == 2 && tm >= 3 && splits == 1;
     const double crowd = roomy ? 0.2 : q4_tall ? 0.3 : 0.56;
     const double round = q4_tall ? 1.25 : 1.56;
