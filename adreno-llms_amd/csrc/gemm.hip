@@ -855,6 +855,268 @@ bool launch_any(int tm, hipStream_t s, int M, int N, int K, const void* x, const
 
 }  // namespace wide
 
+// ---- 256 x 256 blocks, 128 x 128 per wavefront (int8 weights) --------------------------------------
+//
+// The wide kernel above gives a wavefront 64 rows of W against up to 160 rows of x: per MFMA it reads
+// (2 + 2 TM) / (4 TM) fragments from LDS, and at 160 rows that traffic (133 KB per stage of K = 64) takes
+// the LDS four fifths as long as the MFMAs take the matrix cores, overlapped by less than half.  Here the
+// four wavefronts sit two along x by two along W and each owns 128 x 128 of the block's 256 x 256 outputs:
+// sixteen 32 x 32 accumulators (all 256 AGPRs), four fragments of W and four of x per 16 MFMAs, 37 % less
+// LDS read traffic and 19 % less fill traffic per MFMA.  Same LDS layout, swizzles, K permutation, fills
+// and barrier scheme as the wide kernel; three stages of 48 KB.  It needs whole rounds of 256-row tiles to
+// pay: a few hundred tiles at least, and a long K (each block's prologue and epilogue stand alone on its CU).
+namespace quad {
+
+constexpr int kBM = 256, kBN = 256, kStages = 3;
+constexpr int kXStage = kBM * 128, kWStage = kBN * 64, kStage = kXStage + kWStage;
+constexpr int kXLoads = 8, kWLoads = 4, kLoads = kXLoads + kWLoads;   // 1 KB loads per wavefront and stage
+constexpr int kReads = 12, kConv = 16, kMfmas = 32;                   // per half stage (K = 32)
+constexpr int kERow = 272;                                            // epilogue: 128 columns of fp16 + 16 bytes
+
+struct Frags {
+    u32x4 w[4];                // 16 int8 weights of four 32-row fragments of W
+    uint32_t wf[4][2][4];      // the same as fp16: [fragment][MFMA of the pair][4 dwords = 8 halves]
+    u32x4 x[2][4];             // [MFMA of the pair][32-row fragment of x]
+};
+
+using wide::lds_fill16;
+using wide::static_for;
+using wide::pack_half2;
+
+__global__ __launch_bounds__(256) void gemm_quad(const uint16_t* __restrict__ X, const uint8_t* __restrict__ W,
+                                                 const uint16_t* __restrict__ scale, uint16_t* __restrict__ out,
+                                                 int M, int N, int K) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wr = w >> 1, wc = w & 1;                  // this wavefront's 128 rows of x, 128 rows of W
+    const int g = lane >> 5, li = lane & 31;
+    // block -> tile: as in the wide kernel (an XCD takes a contiguous eighth of the list, bands of 4 tiles along N)
+    int tile_m, tile_n;
+    {
+        const int tiles_m = (M + kBM - 1) / kBM, tiles_n = (N + kBN - 1) / kBN, total = tiles_m * tiles_n;
+        const int per_xcd = (total + 7) / 8;
+        const int l = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+        if (blockIdx.x >= 8 * per_xcd || l >= total) return;          // whole block, before any barrier
+        constexpr int kBand = 4;
+        const int band = l / (kBand * tiles_m);
+        const int width = tiles_n - band * kBand < kBand ? tiles_n - band * kBand : kBand;
+        const int in_band = l - band * kBand * tiles_m;
+        tile_m = in_band / width;
+        tile_n = band * kBand + in_band % width;
+    }
+    const int m0 = tile_m * kBM, n0 = tile_n * kBN;
+    const uint32_t lbase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((wide::lds_u8*)lds));
+
+    // fill side: x load j covers rows 8 (w + 4 j) .. + 7 of the tile (128 bytes each, chunk p of row r in slot
+    // p ^ ((r >> 1) & 7)); W load j rows 16 (4 w + j) .. + 15 (64 bytes each, slot p ^ ((r >> 2) & 3))
+    uint32_t xsrc[kXLoads], wsrc[kWLoads];
+    #pragma unroll
+    for (int j = 0; j < kXLoads; ++j) {
+        const int r = 8 * (w + 4 * j) + (lane >> 3);
+        const int c = (lane & 7) ^ ((r >> 1) & 7);
+        const int m = m0 + r < M ? m0 + r : M - 1;
+        xsrc[j] = static_cast<uint32_t>(m) * K * 2u + c * 16u;
+    }
+    #pragma unroll
+    for (int j = 0; j < kWLoads; ++j) {
+        const int r = 16 * (4 * w + j) + (lane >> 2);
+        const int c = (lane & 3) ^ ((r >> 2) & 3);
+        const int n = n0 + r < N ? n0 + r : N - 1;
+        wsrc[j] = static_cast<uint32_t>(n) * K + c * 16u;
+    }
+    const uint8_t* Xb = reinterpret_cast<const uint8_t*>(X);
+    auto fill_one = [&](int stage_k, int slot, auto jc) {
+        constexpr int j = decltype(jc)::value;
+        uint8_t* xs = lds + slot * kStage;
+        if constexpr (j < kXLoads)
+            lds_fill16(Xb + static_cast<size_t>(stage_k) * 128 + xsrc[j], xs + 1024 * (w + 4 * j));
+        else
+            lds_fill16(W + static_cast<size_t>(stage_k) * 64 + wsrc[j - kXLoads], xs + kXStage + 1024 * (4 * w + (j - kXLoads)));
+    };
+    auto fill_stage = [&](int stage_k, int slot) {
+        static_for<kLoads>([&](auto jc) { fill_one(stage_k, slot, jc); });
+    };
+
+    // read side: pair S of a stage, MFMA e of the pair: x chunk 4 S + 2 g + e, W chunk 2 S + g
+    const uint32_t xrow = lbase + (128u * wr + li) * 128u, xq = (2u * g) ^ ((li >> 1) & 7u);
+    const uint32_t wrow = lbase + kXStage + (128u * wc + li) * 64u, wq = g ^ ((li >> 2) & 3u);
+    uint32_t xoff[2][2], woff[2];
+    #pragma unroll
+    for (int S = 0; S < 2; ++S) {
+        #pragma unroll
+        for (int e = 0; e < 2; ++e) xoff[S][e] = xrow + (((4u * S + e) ^ xq) << 4);
+        woff[S] = wrow + (((2u * S) ^ wq) << 4);
+    }
+    // read j of a set: the four W fragments first, then x for the first and the second MFMA of the pair
+    auto read_one = [&](Frags& F, uint32_t slot_bytes, auto Sc, auto jc) {
+        constexpr int S = decltype(Sc)::value, j = decltype(jc)::value;
+        if constexpr (j < 4) {
+            const uint32_t a = woff[S] + slot_bytes;
+            MI_LDS_READ16(F.w[j], a, j * 32 * 64);
+        } else {
+            constexpr int e = (j - 4) / 4, t = (j - 4) % 4;
+            const uint32_t a = xoff[S][e] + slot_bytes;
+            MI_LDS_READ16(F.x[e][t], a, t * 4096);
+        }
+    };
+    auto convert_one = [&](Frags& F, auto jc) {
+        constexpr int j = decltype(jc)::value, u = j / 4, d = j % 4;
+        i8x4_to_h4(F.w[u][d], F.wf[u][d / 2][2 * (d % 2)], F.wf[u][d / 2][2 * (d % 2) + 1]);
+    };
+
+    floatx16 acc[4][4];
+    #pragma unroll
+    for (int u = 0; u < 4; ++u)
+        #pragma unroll
+        for (int t = 0; t < 4; ++t)
+            #pragma unroll
+            for (int r = 0; r < 16; ++r) acc[u][t][r] = 0.0f;
+
+    auto mfma_one = [&](const Frags& F, auto nc) {
+        constexpr int n = decltype(nc)::value, e = n / 16, u = (n / 4) % 4, t = n % 4;
+        const u32x4 wv = u32x4{F.wf[u][e][0], F.wf[u][e][1], F.wf[u][e][2], F.wf[u][e][3]};
+        acc[u][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, wv),
+                                                          __builtin_bit_cast(half8, F.x[e][t]), acc[u][t], 0, 0, 0);
+    };
+
+    // one half stage: the fills of a later stage, the reads and conversions of the next fragments, dealt out
+    // between the MFMAs of the current ones
+    auto half_stage = [&](Frags& C, Frags& Nx, uint32_t next_bytes, auto NSc, auto fillc, int fill_k, int fill_slot) {
+        constexpr bool FILL = decltype(fillc)::value;
+        constexpr int nF = FILL ? kLoads : 0;
+        constexpr int A = nF + kReads + 1 + kConv;
+        static_for<kMfmas>([&](auto nc) {
+            constexpr int n = decltype(nc)::value;
+            mfma_one(C, nc);
+            MI_SCHED_FENCE();
+            constexpr int a0 = n * A / kMfmas, a1 = (n + 1) * A / kMfmas;
+            static_for<a1 - a0>([&](auto kc) {
+                constexpr int a = a0 + decltype(kc)::value;
+                if constexpr (a < nF) {
+                    fill_one(fill_k, fill_slot, std::integral_constant<int, a>{});
+                } else if constexpr (a < nF + kReads) {
+                    read_one(Nx, next_bytes, NSc, std::integral_constant<int, a - nF>{});
+                } else if constexpr (a == nF + kReads) {
+                    // LDS returns in order: with the eight x reads outstanding, the four W reads are back
+                    asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(Nx.w[0]), "+v"(Nx.w[1]), "+v"(Nx.w[2]), "+v"(Nx.w[3]) : : "memory");
+                    MI_SCHED_FENCE();
+                } else {
+                    convert_one(Nx, std::integral_constant<int, a - nF - kReads - 1>{});
+                }
+            });
+            MI_SCHED_FENCE();
+        });
+        MI_WAIT_LGKM(0);
+        MI_SCHED_FENCE();
+    };
+    // at most `stages` (0 or 1) of this wavefront's stage fills still in flight
+    auto wait_fills = [&](int stages) {
+        if (stages >= 1) MI_WAIT_VM(kLoads); else MI_WAIT_VM(0);
+    };
+
+    const int nk = K / 64;
+    Frags FA, FB;
+    #pragma unroll
+    for (int st = 0; st < kStages - 1; ++st)
+        if (st < nk) fill_stage(st, st);
+    wait_fills((nk < kStages - 1 ? nk : kStages - 1) - 1);          // stage 0 has landed
+    __builtin_amdgcn_s_barrier();
+    MI_SCHED_FENCE();
+    static_for<kReads>([&](auto jc) { read_one(FA, 0u, std::integral_constant<int, 0>{}, jc); });
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(FA.w[0]), "+v"(FA.w[1]), "+v"(FA.w[2]), "+v"(FA.w[3]) : : "memory");
+    MI_SCHED_FENCE();
+    static_for<kConv>([&](auto jc) { convert_one(FA, jc); });
+
+    auto stage = [&](int i, int slot, auto fillc) {
+        const int next = slot + 1 == kStages ? 0 : slot + 1;
+        const int prev = slot == 0 ? kStages - 1 : slot - 1;
+        half_stage(FA, FB, static_cast<uint32_t>(slot) * kStage, std::integral_constant<int, 1>{}, std::false_type{}, 0, 0);
+        MI_SCHED_FENCE();
+        const int last = i + kStages - 2 < nk - 1 ? i + kStages - 2 : nk - 1;   // newest stage requested so far
+        wait_fills(last - (i + 1));
+        __builtin_amdgcn_s_barrier();
+        MI_SCHED_FENCE();
+        half_stage(FB, FA, static_cast<uint32_t>(next) * kStage, std::integral_constant<int, 0>{}, fillc, i + kStages - 1, prev);
+        MI_SCHED_FENCE();
+    };
+    int slot = 0, i = 0;
+    for (; i + kStages - 1 < nk; ++i) {
+        stage(i, slot, std::true_type{});
+        slot = slot + 1 == kStages ? 0 : slot + 1;
+    }
+    for (; i < nk; ++i) {
+        stage(i, slot, std::false_type{});
+        slot = slot + 1 == kStages ? 0 : slot + 1;
+    }
+
+    // epilogue: D[i][j], i = 8 (r / 4) + 4 g + r % 4 a row of W (an output column), j = li a row of x.  The scaled
+    // fp16 values go through LDS (this wavefront's own 128 x 128 patch, rows padded to 272 bytes) so that the
+    // stores are 16 bytes per lane, 256 consecutive bytes per 16 lanes.
+    MI_WAIT_LGKM(0);
+    __builtin_amdgcn_s_barrier();                        // nobody reads operands from LDS any more
+    MI_SCHED_FENCE();
+    uint8_t* ebase = lds + w * (128 * kERow);
+    const bool cols4 = (N % 4) == 0 && reinterpret_cast<uintptr_t>(scale) % 8 == 0;
+    #pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        #pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+            const int nq = n0 + 128 * wc + 32 * u + 8 * rq + 4 * g;
+            uint32_t h[4];
+            if (cols4 && nq + 3 < N) {
+                const uint2 v = *reinterpret_cast<const uint2*>(scale + nq);
+                h[0] = v.x & 0xFFFFu; h[1] = v.x >> 16; h[2] = v.y & 0xFFFFu; h[3] = v.y >> 16;
+            } else {
+                #pragma unroll
+                for (int e = 0; e < 4; ++e) h[e] = scale[nq + e < N ? nq + e : N - 1];
+            }
+            float s4[4];
+            #pragma unroll
+            for (int e = 0; e < 4; ++e) s4[e] = __half2float(__ushort_as_half(static_cast<uint16_t>(h[e])));
+            #pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t lo = pack_half2(acc[u][t][4 * rq] * s4[0], acc[u][t][4 * rq + 1] * s4[1]);
+                const uint32_t hi = pack_half2(acc[u][t][4 * rq + 2] * s4[2], acc[u][t][4 * rq + 3] * s4[3]);
+                *reinterpret_cast<uint2*>(ebase + (32 * t + li) * kERow + (32 * u + 8 * rq + 4 * g) * 2) = uint2{lo, hi};
+            }
+        }
+    }
+    // each wavefront reads back only what it wrote itself
+    const int ncol = n0 + 128 * wc + 8 * (lane & 15);    // first of this lane's 8 output columns
+    const bool cols8 = (N % 8) == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    #pragma unroll 4
+    for (int j = 0; j < 32; ++j) {
+        const int row = 4 * j + (lane >> 4);
+        const u32x4 v = *reinterpret_cast<const u32x4*>(ebase + row * kERow + (lane & 15) * 16);
+        const int m = m0 + 128 * wr + row;
+        if (m >= M) continue;
+        uint16_t* dst = out + static_cast<size_t>(m) * N + ncol;
+        if (cols8 && ncol + 7 < N) {
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
+        } else {
+            #pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (ncol + e < N) dst[e] = static_cast<uint16_t>(v[e / 2] >> (16 * (e % 2)));
+        }
+    }
+}
+
+bool launch(hipStream_t s, int M, int N, int K, const void* x, const void* W, const void* scale, void* out) {
+    constexpr size_t lds_bytes = static_cast<size_t>(kStages) * kStage;
+    static_assert(4 * 128 * kERow <= kStages * kStage, "the epilogue's patches fit the operand stages");
+    if (!MI_ONCE_OK(MI_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_quad),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes))))
+        return false;
+    const long total = static_cast<long>((N + kBN - 1) / kBN) * ((M + kBM - 1) / kBM);
+    hipLaunchKernelGGL(gemm_quad, dim3(static_cast<unsigned>(8 * ((total + 7) / 8))), dim3(256), lds_bytes, s,
+                       static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(W),
+                       static_cast<const uint16_t*>(scale), static_cast<uint16_t*>(out), M, N, K);
+    return MI_HIP_OK(hipGetLastError());
+}
+
+}  // namespace quad
+
 // ---- a few rows of x (M <= 64): the weights stream once, as in the GEMV ------------------------
 //
 // With up to 64 rows of x the contraction is bound by the weights' bytes, like the GEMV, not by
@@ -1398,6 +1660,19 @@ GemmPlan plan_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, size_t w
         p.kernel = 1; p.tile_rows = 32 * tm; p.k_slices = splits;
         return p;
     }
+    // The 256 x 256 blocks (int8 weights): by name (mode 30), or by themselves where they pay, which takes
+    // several full rounds of such tiles and a long K.  Measured against the 160-row wide tiles: 8192 x 8192 x
+    // 8192 884 against 968 us, 8192 x 8192 x 2048 247 against 264 us; but 4096 x 4864 x 4864 (304 tiles, 1.2
+    // rounds) 229 against 177 us and 4096 x 9728 x 896 (K of 14 stages) 89 against 78 us.
+    if (kind == WK_I8 && wide_fits && (mode == 30 || mode == 0)) {
+        const long t256 = static_cast<long>((M + 255) / 256) * ((N + 255) / 256);
+        const long rounds = (t256 + cus - 1) / cus;
+        if (mode == 30 || (K >= 2048 && rounds >= 4 && t256 * 10 >= rounds * cus * 9)) {
+            p.kernel = 5; p.tile_rows = 256;
+            return p;
+        }
+    }
+    if (mode == 30) return p;
     // int8 and fp16, a few rows of x: the streaming kernel (mode 5 asks for it by name, up to 64 rows)
     if (M <= skinny::kMaxM && (mode == 5 || (mode == 0 && skinny::preferred(kind, M, N, K, cus, workspace_bytes)))) {
         const skinny::Shape sh = skinny::pick_shape(kind, M, N, K, cus, workspace_bytes);
@@ -1454,6 +1729,7 @@ bool launch_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, const void
             return kind == WK_F16 ? skinny::launch<WK_F16, 1>(s, M, N, K, x, W, scale, out, sh, workspace, ws_bytes)
                                   : skinny::launch<WK_I8, 1>(s, M, N, K, x, W, scale, out, sh, workspace, ws_bytes);
         }
+        case 5: return quad::launch(s, M, N, K, x, W, scale, out);
         case 2: return launch_tile<64, 64, 32, 32>(s, kind, M, N, K, x, W, scale, out);
         case 3: return launch_tile<128, 128, 64, 64>(s, kind, M, N, K, x, W, scale, out);
         default:

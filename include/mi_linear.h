@@ -178,7 +178,8 @@ int   mi_graph_destroy(void* graph);
  * the same tolerance, only the speed differs): 2 = the 64 x 64 tile kernel (int8 and fp16
  * weights; fails for Q4), 3 = the wide kernel, 10 + t (t = 1..5) = the wide kernel with 32 t
  * rows of x per block, 100 s + 10 + t (s = 1..24) = the same with K cut into s slices (refused where the
- * slices' fp32 sums do not fit the stream's workspace), 5 = the streaming kernel for up to 64 rows of x (every kind of weights takes
+ * slices' fp32 sums do not fit the stream's workspace), 30 = the kernel with 256 x 256 blocks (int8 weights only; mode 0
+ * takes it by itself for contractions of several rounds of such blocks at K >= 2048), 5 = the streaming kernel for up to 64 rows of x (every kind of weights takes
  * it by itself in mode 0 up to 32 to 64 rows, depending on the shape, where it is the faster one;
  * fails for more than 64 rows).
  * Q4 weights: a weight q * scale (4 and 11 significant bits) is not an fp16 number in general.
@@ -209,7 +210,7 @@ int mi_stream_set_modes(void* stream, int gemv_mode, int gemm_mode);
  * reduction launch), 2 / 3 = the 64 x 64 / 128 x 128 tile kernel, 4 = the streaming kernel for up
  * to 64 rows of x (*tile_rows = M rounded up to 16, *k_slices = wavefronts, over one or several
  * blocks, that share one strip of 16 rows of W; slices over several blocks also end in a reduction
- * launch), -1 = bad arguments.  For tests and tuning; tile_rows and k_slices
+ * launch), 5 = the MFMA kernel with 256 x 256 blocks (int8 weights), -1 = bad arguments.  For tests and tuning; tile_rows and k_slices
  * may be NULL. */
 int mi_linear_plan(void* stream, int M, int N, int K, const void* x, const void* W, int* tile_rows, int* k_slices);
 

@@ -36,7 +36,7 @@ def _ulp_apart(a_u16, b_u16):
 def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0, plan=None):
     """tile is the mi_set_gemm_mode value: 0 = the library's own choice, 1 = rows of GEMV,
     2 = the 64 x 64 MFMA kernel, 3 = the wide kernel with its own choice of rows of x per
-    block, 4 = Q4 weights rounded to fp16 once, 5 = the streaming kernel for up to 64 rows of x,
+    block, 30 = the kernel with 256 x 256 blocks (int8), 4 = Q4 weights rounded to fp16 once, 5 = the streaming kernel for up to 64 rows of x,
     11..15 = the wide kernel with 32, 64, .. 160 rows of x per block.  plan: a list that receives (kernel, rows of x per block, slices of K) of the call."""
     xb, wb = mil.Buffer.from_host(X), mil.Buffer.from_host(W_host)
     sb = mil.Buffer.from_host(scale_host) if scale_host is not None else None
@@ -61,7 +61,7 @@ def _gemm(queue, M, N, K, X, W_host, scale_host, kind, tile=0, plan=None):
     return full[pad:-pad].reshape(M, N)
 
 
-@pytest.mark.parametrize("tile", [0, 2, 3, 11, 12, 13, 14, 15])
+@pytest.mark.parametrize("tile", [0, 2, 3, 11, 12, 13, 14, 15, 30])
 @pytest.mark.parametrize("M", [16, 64, 100, 512])
 @pytest.mark.parametrize("N,K", [(4864, 896), (896, 4864), (200, 128), (130, 576), (131, 64)])
 def test_int8_gemm_matches_rows_of_gemv(queue, M, N, K, tile):
@@ -102,7 +102,7 @@ def test_fp16_gemm_exact_and_repeatable_on_integer_data(queue, tile):
         assert np.array_equal(got.view(np.float16), want)
 
 
-@pytest.mark.parametrize("tile", [2, 3, 11, 13, 15])
+@pytest.mark.parametrize("tile", [2, 3, 11, 13, 15, 30])
 def test_gemm_exact_on_integer_data(queue, tile):
     # small integers: every partial sum is exact in fp32, so any summation order gives the same bits
     rng = np.random.default_rng(3)
@@ -116,7 +116,7 @@ def test_gemm_exact_on_integer_data(queue, tile):
     assert np.array_equal(got, O.gemm_i8(X, q, s.view(np.uint16)))
 
 
-@pytest.mark.parametrize("tile", [2, 3, 12, 14, 15])
+@pytest.mark.parametrize("tile", [2, 3, 12, 14, 15, 30])
 def test_gemm_unit_rows_pick_weight_columns(queue, tile):
     # x rows are unit vectors: out[i, :] must be the dequantised column k_i of W (index check)
     M, N, K = 64, 320, 896
@@ -130,7 +130,7 @@ def test_gemm_unit_rows_pick_weight_columns(queue, tile):
     assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("tile", [2, 11, 12, 13, 14, 15])
+@pytest.mark.parametrize("tile", [2, 11, 12, 13, 14, 15, 30])
 def test_gemm_repeats_identically(queue, tile):
     """The same launch 25 times: every result identical to the first and within tolerance of the
     oracle (a race between the LDS fills, the fragment reads and the barriers would show here)."""
@@ -154,6 +154,44 @@ def test_gemm_repeats_identically(queue, tile):
     for i, ob in enumerate(outs[1:]):
         assert np.array_equal(ob.read(np.uint16, (M, N)), first), f"launch {i + 1} differs from launch 0"
     mil.nnopt_unregister_weight(wb)
+
+
+def test_the_256_row_blocks_give_the_wide_kernels_bits_and_are_the_choice_for_large_contractions(queue):
+    """The kernel with 256 x 256 blocks (128 x 128 per wavefront) feeds every output element the same K-stages
+    in the same order as the wide kernel, so the two agree bit for bit: ragged shapes with partial blocks in
+    both directions (mode 30 against mode 15, guard words intact), then a contraction large enough for the
+    library to take the kernel by itself (8192 x 8192 x 2048: 1024 blocks, four rounds), whose plan is checked
+    and whose output is compared with the wide kernel's through a row sample and a checksum of every row."""
+    for (M, N, K) in ((700, 1300, 2112), (257, 255, 64), (1024, 1024, 2048), (3, 600, 128)):
+        print(f"256-row blocks M={M} N={N} K={K}", flush=True)
+        W, X = synth_w(960 + M, N, K), synth_x(961 + M, M, K)
+        q, s = mil.quantize_int8(W)
+        plan = []
+        got = _gemm(queue, M, N, K, X, q, s, "i8", 30, plan=plan)
+        assert plan[0][0] == 5 and plan[0][1] == 256, plan
+        assert np.array_equal(got, _gemm(queue, M, N, K, X, q, s, "i8", 15))
+    M, N, K = 8192, 8192, 2048
+    print(f"256-row blocks M={M} N={N} K={K}, the library's own choice", flush=True)
+    W, X = synth_w(970, N, K), synth_x(971, M, K)
+    q, s = mil.quantize_int8(W)
+    xb, wb, sb = mil.Buffer.from_host(X), mil.Buffer.from_host(q), mil.Buffer.from_host(s)
+    assert mil.nnopt_register_int8_weight(wb, sb, N, K)
+    outs = []
+    try:
+        assert mil.linear_plan(queue, M, N, K, xb, wb)[0] == 5
+        for mode in (0, 15):
+            ob = mil.Buffer(M * N * 2)
+            mil.lib().mi_set_gemm_mode(mode)
+            assert mil.pytorch_linear(queue, M, N, K, xb, wb, ob)
+            queue.finish()
+            outs.append(ob.read(np.uint16, (M, N)))
+    finally:
+        mil.lib().mi_set_gemm_mode(0)
+        mil.nnopt_unregister_weight(wb)
+    assert np.array_equal(outs[0], outs[1])
+    rows = [0, 255, 256, 4097, 8191]                     # and against the oracle, on a few rows
+    want = O.gemm_i8(X[rows], q, s.view(np.uint16))
+    assert _ulp_apart(outs[0][rows], want).max() <= 1
 
 
 # ---- up to 64 rows of x: the kernel that streams W once (mode 5; mode 0 picks it by itself) ----
