@@ -445,6 +445,29 @@ def main():
         detail[f"c5_int8_gemm_M16_N{VOCAB}_K{H}"] = {
             "us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
             "frac_hbm": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        # a large square contraction (no config asks for it): the MFMA main loop without the short K of the
+        # configured shapes; the library's own choice (256 x 256 blocks) and the 160-row wide tiles
+        Mq = Nq = Kq = 8192
+        qh, sh = mil.quantize_int8(mil.synth_normal_f16(79, 0.02, (Nq, Kq)))
+        wb, sb = mil.Buffer.from_host(qh), mil.Buffer.from_host(sh)
+        assert mil.nnopt_register_int8_weight(wb, sb, Nq, Kq)
+        xb = mil.Buffer.from_host(mil.synth_normal_f16(80, 1.0, (Mq, Kq)))
+        ob = mil.Buffer(Mq * Nq * 2)
+        arr = mil.make_calls([(Mq, Nq, Kq, xb, wb, ob)] * 3)
+        for mode, tag in ((0, "proxy_int8_gemm_M8192_N8192_K8192"), (15, "proxy_int8_gemm_M8192_N8192_K8192_160_row_tiles")):
+            mil.lib().mi_set_gemm_mode(mode)
+            try:
+                kern, rows, slices = mil.linear_plan(queue, Mq, Nq, Kq, xb, wb)
+                mil.linear_batch(queue, arr)
+                ms = time_region(mil, queue, lambda: mil.linear_batch(queue, arr), 1, 5) / 3
+            finally:
+                mil.lib().mi_set_gemm_mode(0)
+            flop = 2.0 * Mq * Nq * Kq
+            detail[tag] = {"kernel": {1: "wide", 5: "blocks256"}.get(kern, str(kern)), "rows_of_x_per_block": rows,
+                           "us": round(ms * 1e3, 1), "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 1),
+                           "frac_mfma_fp16_peak": round(flop / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)}
+        mil.nnopt_unregister_weight(wb)
+        del xb, ob, wb, sb
         # the same contractions with fp16 weights
         for (N, K) in ((INTER, H), (H, INTER)):
             wb = mil.Buffer.from_host(mil.synth_normal_f16(77, 0.02, (N, K)))
