@@ -303,7 +303,7 @@ def pytorch_linear_argmax(queue, N, K, x, W, logits, token_out, num_partials=32)
 
 def linear_plan(queue, M, N, K, x, W):
     """(kernel, rows of x per block, slices of K) mi_linear would use; kernel 0 = GEMV rows, 1 = wide MFMA kernel,
-    2 / 3 = tile kernels, 4 = the streaming kernel for up to 64 rows of x."""
+    2 / 3 = tile kernels, 4 = the streaming kernel for up to 64 rows of x, 5 = the kernel with 256 x 256 blocks."""
     tr, ks = C.c_int(0), C.c_int(1)
     kern = lib().mi_linear_plan(_q(queue), M, N, K, _h(x), _h(W), C.byref(tr), C.byref(ks))
     return kern, tr.value, ks.value

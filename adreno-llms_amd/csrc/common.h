@@ -126,7 +126,8 @@ double gemm_estimate_us(WeightKind kind, int M, int N, int K, size_t workspace_b
 // What launch_gemm would run for this call on this stream: kernel 1 = the wide kernel (tile_rows
 // rows of x per block, K in k_slices slices, `terms` fp16 terms per Q4 weight), 2 / 3 = 64 x 64 /
 // 128 x 128 tiles, 4 = the streaming kernel for up to 64 rows of x (k_slices wavefronts of a block
-// share a strip of W); kernel -1 = a mode that cannot serve this call.
+// share a strip of W), 5 = the kernel with 256 x 256 blocks (int8 weights); kernel -1 = a mode that
+// cannot serve this call.
 struct GemmPlan { int kernel = -1, tile_rows = 0, k_slices = 1, terms = 1; };
 GemmPlan plan_gemm(hipStream_t s, WeightKind kind, int M, int N, int K, size_t workspace_bytes);
 // workspace: device memory that belongs to stream s (or null): the wide kernel may cut K into
